@@ -1,0 +1,57 @@
+"""Builds libsage_mi355x.so (the gfx950 HIP kernels and their C ABI) in-tree with hipcc.
+
+Run as ``python -m baselinebenchmark_amd.build``.  The library lands next to the sources in
+``baselinebenchmark_amd/csrc/`` where ``_cabi.py`` loads it from; nothing is built lazily at
+import time, so a missing library is a loud error.
+"""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+from pathlib import Path
+
+CSRC = Path(__file__).resolve().parent / "csrc"
+LIB = CSRC / "libsage_mi355x.so"
+SOURCES = ["sage_quant.hip", "sage_attn.hip", "sage_api.hip"]
+FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
+    # correctly rounded fp32 divide (the INT8 quantiser's contract) and no packed-fp32 selection
+    "-fhip-fp32-correctly-rounded-divide-sqrt",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+
+
+def _hipcc() -> str:
+    return os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+
+
+def _compile(src: str) -> Path:
+    obj = CSRC / (src.replace(".hip", ".o"))
+    cmd = [_hipcc(), *FLAGS, "-c", str(CSRC / src), "-o", str(obj)]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    noise = "is not a recognized feature for this target"
+    err = "\n".join(l for l in res.stderr.splitlines() if noise not in l)
+    if res.returncode != 0:
+        raise RuntimeError(f"hipcc failed for {src}:\n{err}")
+    if err.strip():
+        print(err, file=sys.stderr)
+    return obj
+
+
+def build(verbose: bool = True) -> Path:
+    with ThreadPoolExecutor(max_workers=len(SOURCES)) as ex:
+        objs = list(ex.map(_compile, SOURCES))
+    cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", *map(str, objs), "-o", str(LIB)]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"link failed:\n{res.stderr}")
+    if verbose:
+        print(f"built {LIB} ({LIB.stat().st_size} bytes)")
+    return LIB
+
+
+if __name__ == "__main__":
+    build()

@@ -1,0 +1,308 @@
+// C ABI of libsage_mi355x.so (declared in include/sage_mi355x.h): argument validation with the
+// reference's error classes, workspace carving, the one-call sageattn pipeline and the launch
+// geometry of every kernel.  Nothing here allocates device memory or synchronises.
+#include "sage_launch.h"
+#include "../../include/sage_mi355x.h"
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <cmath>
+
+using namespace sage;
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int hip_fail(hipError_t e, const char* what) {
+  return fail(SAGE_ELAUNCH, "%s: %s", what, hipGetErrorString(e));
+}
+
+inline size_t align_up(size_t x, size_t a = 256) { return (x + a - 1) / a * a; }
+
+bool valid_blk_quant(int blk) { return blk == 16 || blk == 32 || blk == 64 || blk == 128; }
+
+int check_common(int B, int H, int L, int D, int dtype) {
+  if (B < 0 || H < 0 || L < 0) return fail(SAGE_EINVAL, "negative dimension (B=%d H=%d L=%d)", B, H, L);
+  if (D != 64 && D != 128) return fail(SAGE_ENOTIMPL, "head_dim %d is not supported (64 or 128)", D);
+  if (dtype != SAGE_DT_F16 && dtype != SAGE_DT_BF16) return fail(SAGE_ETYPE, "dtype flag %d is not fp16(0)/bf16(1)", dtype);
+  return SAGE_OK;
+}
+
+int check_stride16(const char* name, int64_t sb, int64_t sh, int64_t sn, int esz, const void* p) {
+  // 128-bit accesses: every row must start on a 16-byte boundary
+  if ((sb * esz) % 16 || (sh * esz) % 16 || (sn * esz) % 16 || (reinterpret_cast<uintptr_t>(p) % 16))
+    return fail(SAGE_EINVAL, "%s: base pointer and strides must be 16-byte aligned", name);
+  return SAGE_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* sage_backend_name(void) { return "mi355x_hip_int8_qk_fp8_fp16_pv"; }
+
+const char* sage_last_error(void) { return g_err; }
+
+int sage_quant_int8(const void* x, int8_t* out, float* scale, const void* km, int B, int H, int L, int D, int64_t x_sb,
+                    int64_t x_sh, int64_t x_sn, int64_t o_sb, int64_t o_sh, int64_t o_sn, int64_t km_sb, int64_t km_sh,
+                    int blk, float mult, int dtype, const int32_t* cu_seqlens, const int32_t* cu_blocks,
+                    int64_t scale_sh, sage_stream_t stream) {
+  if (int rc = check_common(B, H, L, D, dtype)) return rc;
+  if (!valid_blk_quant(blk)) return fail(SAGE_ENOTIMPL, "quantisation block %d is not supported (16, 32, 64, 128)", blk);
+  if (B == 0 || H == 0 || L == 0) return SAGE_OK;
+  if (!x || !out || !scale) return fail(SAGE_EINVAL, "null tensor pointer");
+  if (cu_seqlens && !cu_blocks) return fail(SAGE_EINVAL, "packed mode needs cu_blocks");
+  if (int rc = check_stride16("x", x_sb, x_sh, x_sn, 2, x)) return rc;
+  if (int rc = check_stride16("out", o_sb, o_sh, o_sn, 1, out)) return rc;
+  if ((o_sn % 8) || (o_sh % 8) || (o_sb % 8)) return fail(SAGE_EINVAL, "out strides must be multiples of 8");
+  if (km && int(check_stride16("km", km_sb, km_sh, 0, 2, km))) return SAGE_EINVAL;
+  QuantArgs a;
+  a.x = (const u16*)x; a.out = out; a.scale = scale; a.km = (const u16*)km;
+  a.B = B; a.H = H; a.L = L; a.D = D;
+  a.x_sb = x_sb; a.x_sh = x_sh; a.x_sn = x_sn; a.o_sb = o_sb; a.o_sh = o_sh; a.o_sn = o_sn;
+  a.km_sb = km_sb; a.km_sh = km_sh; a.blk = blk; a.mult = mult;
+  a.cu_seqlens = cu_seqlens; a.cu_blocks = cu_blocks; a.scale_sh = scale_sh;
+  hipError_t e = launch_quant_int8(a, dtype, (L + blk - 1) / blk, (hipStream_t)stream);
+  if (e != hipSuccess) return hip_fail(e, "sage_quant_int8");
+  return SAGE_OK;
+}
+
+size_t sage_k_mean_workspace_bytes(int B, int H, int L, int D) {
+  return align_up((size_t)B * H * colstat_chunks(L) * D * sizeof(double));
+}
+
+int sage_k_mean(const void* k, void* km, void* workspace, size_t workspace_bytes, int B, int H, int L, int D, int64_t k_sb,
+                int64_t k_sh, int64_t k_sn, int dtype, const int32_t* cu_seqlens, sage_stream_t stream) {
+  if (int rc = check_common(B, H, L, D, dtype)) return rc;
+  if (B == 0 || H == 0) return SAGE_OK;
+  if (!k || !km || !workspace) return fail(SAGE_EINVAL, "null tensor pointer");
+  if (workspace_bytes < sage_k_mean_workspace_bytes(B, H, L, D)) return fail(SAGE_EWORKSPACE, "k_mean workspace too small");
+  if (int rc = check_stride16("k", k_sb, k_sh, k_sn, 2, k)) return rc;
+  ColStatArgs a;
+  a.x = (const u16*)k; a.partial = workspace; a.B = B; a.H = H; a.L = L; a.D = D;
+  a.x_sb = k_sb; a.x_sh = k_sh; a.x_sn = k_sn; a.nchunk = colstat_chunks(L); a.cu_seqlens = cu_seqlens;
+  if (a.nchunk == 0) a.nchunk = 1;  // L == 0: the finalize kernel still writes zeros
+  hipError_t e = launch_k_mean(a, dtype, km, (hipStream_t)stream);
+  if (e != hipSuccess) return hip_fail(e, "sage_k_mean");
+  return SAGE_OK;
+}
+
+size_t sage_prep_v_workspace_bytes(int B, int H, int L, int D, int pv_mode) {
+  if (pv_mode != SAGE_PV_FP8) return 0;
+  int nc = colstat_chunks(L);
+  return align_up((size_t)B * H * (nc ? nc : 1) * D * sizeof(float));
+}
+
+size_t sage_v_panel_bytes(int B, int H, int L, int D, int pv_mode) {
+  size_t np = (L + SAGE_PANEL_ROWS - 1) / SAGE_PANEL_ROWS;
+  return (size_t)B * H * np * SAGE_PANEL_ROWS * D * (pv_mode == SAGE_PV_FP8 ? 1 : 2);
+}
+
+int sage_prep_v(const void* v, void* panels, float* v_scale, void* workspace, size_t workspace_bytes, int B, int H, int L,
+                int D, int64_t v_sb, int64_t v_sh, int64_t v_sn, int dtype, int pv_mode, const int32_t* cu_seqlens,
+                const int32_t* cu_panels, int64_t panel_sh, sage_stream_t stream) {
+  if (int rc = check_common(B, H, L, D, dtype)) return rc;
+  if (pv_mode != SAGE_PV_FP16 && pv_mode != SAGE_PV_FP8) return fail(SAGE_EINVAL, "pv_mode %d unknown", pv_mode);
+  if (B == 0 || H == 0 || L == 0) return SAGE_OK;
+  if (!v || !panels) return fail(SAGE_EINVAL, "null tensor pointer");
+  if (cu_seqlens && !cu_panels) return fail(SAGE_EINVAL, "packed mode needs cu_panels");
+  if (int rc = check_stride16("v", v_sb, v_sh, v_sn, 2, v)) return rc;
+  if (reinterpret_cast<uintptr_t>(panels) % 16) return fail(SAGE_EINVAL, "panels must be 16-byte aligned");
+  hipStream_t st = (hipStream_t)stream;
+  if (pv_mode == SAGE_PV_FP8) {
+    if (!v_scale || !workspace) return fail(SAGE_EINVAL, "fp8 mode needs v_scale and workspace");
+    if (workspace_bytes < sage_prep_v_workspace_bytes(B, H, L, D, pv_mode)) return fail(SAGE_EWORKSPACE, "prep_v workspace too small");
+    ColStatArgs c;
+    c.x = (const u16*)v; c.partial = workspace; c.B = B; c.H = H; c.L = L; c.D = D;
+    c.x_sb = v_sb; c.x_sh = v_sh; c.x_sn = v_sn; c.nchunk = colstat_chunks(L); c.cu_seqlens = cu_seqlens;
+    hipError_t e = launch_v_scale(c, dtype, v_scale, st);
+    if (e != hipSuccess) return hip_fail(e, "sage_prep_v(scale)");
+  }
+  PrepVArgs a;
+  a.v = (const u16*)v; a.panels = (uint8_t*)panels; a.vscale = v_scale; a.B = B; a.H = H; a.L = L; a.D = D;
+  a.v_sb = v_sb; a.v_sh = v_sh; a.v_sn = v_sn; a.cu_seqlens = cu_seqlens; a.cu_panels = cu_panels; a.panel_sh = panel_sh;
+  hipError_t e = launch_prep_v(a, dtype, pv_mode, (L + SAGE_PANEL_ROWS - 1) / SAGE_PANEL_ROWS, st);
+  if (e != hipSuccess) return hip_fail(e, "sage_prep_v");
+  return SAGE_OK;
+}
+
+size_t sage_varlen_plan_ints(int nseq, int total_q) { return (size_t)plan_layout(nseq, total_q).total; }
+
+void sage_varlen_plan_offsets(int nseq, int total_q, int64_t offs[5]) {
+  SagePlanLayout L = plan_layout(nseq, total_q);
+  offs[0] = L.cu_qblk; offs[1] = L.cu_kblk; offs[2] = L.cu_panel; offs[3] = L.ntiles; offs[4] = L.tiles;
+}
+
+int sage_varlen_plan(const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k, int nseq, int total_q, int blkq, int blkk,
+                     int is_causal, int32_t* plan, size_t plan_ints, sage_stream_t stream) {
+  if (nseq <= 0 || nseq > 32767) return fail(SAGE_EINVAL, "number of sequences %d out of range (1..32767)", nseq);
+  if (!cu_seqlens_q || !cu_seqlens_k || !plan) return fail(SAGE_EINVAL, "null pointer");
+  if (!valid_blk_quant(blkq) || !valid_blk_quant(blkk)) return fail(SAGE_ENOTIMPL, "block sizes %d/%d not supported", blkq, blkk);
+  if (plan_ints < sage_varlen_plan_ints(nseq, total_q)) return fail(SAGE_EWORKSPACE, "plan buffer too small");
+  AttnConfig cfg = attn_config(128, 1, true);
+  hipError_t e = launch_varlen_plan(cu_seqlens_q, cu_seqlens_k, nseq, total_q, blkq, blkk, cfg.nw * 32, 64, is_causal, plan,
+                                    (hipStream_t)stream);
+  if (e != hipSuccess) return hip_fail(e, "sage_varlen_plan");
+  return SAGE_OK;
+}
+
+int sage_attn_fwd(const int8_t* q, const int8_t* k, const void* v_panels, const float* q_scale, const float* k_scale,
+                  const float* v_scale, void* out, float* lse, int B, int Hq, int Hkv, int Sq, int Skv, int D, int64_t q_sb,
+                  int64_t q_sh, int64_t q_sn, int64_t k_sb, int64_t k_sh, int64_t k_sn, int64_t o_sb, int64_t o_sh,
+                  int64_t o_sn, int blkq, int blkk, int is_causal, int pv_mode, int out_dtype, const int32_t* cu_seqlens_q,
+                  const int32_t* cu_seqlens_k, const int32_t* plan, int total_q, int64_t q_scale_sh, int64_t k_scale_sh,
+                  int64_t panel_sh, sage_stream_t stream) {
+  if (int rc = check_common(B, Hq, Sq, D, out_dtype)) return rc;
+  if (Hkv <= 0 || Hq % Hkv) return fail(SAGE_EINVAL, "query heads (%d) must be divisible by KV heads (%d)", Hq, Hkv);
+  if (Skv < 0) return fail(SAGE_EINVAL, "negative kv length");
+  if (pv_mode != SAGE_PV_FP16 && pv_mode != SAGE_PV_FP8) return fail(SAGE_EINVAL, "pv_mode %d unknown", pv_mode);
+  if (blkq % 32 || blkk % 32 || blkq <= 0 || blkk <= 0 || blkq > 128 || blkk > 128)
+    return fail(SAGE_ENOTIMPL, "attention needs scale blocks that are multiples of 32 up to 128 (got %d/%d)", blkq, blkk);
+  if (B == 0 || Hq == 0 || Sq == 0) return SAGE_OK;
+  if (!q || !k || !v_panels || !q_scale || !k_scale || !out) return fail(SAGE_EINVAL, "null tensor pointer");
+  if (pv_mode == SAGE_PV_FP8 && !v_scale) return fail(SAGE_EINVAL, "fp8 P.V needs v_scale");
+  if (int rc = check_stride16("q", q_sb, q_sh, q_sn, 1, q)) return rc;
+  if (int rc = check_stride16("k", k_sb, k_sh, k_sn, 1, k)) return rc;
+  if ((o_sb % 4) || (o_sh % 4) || (o_sn % 4) || reinterpret_cast<uintptr_t>(out) % 8)
+    return fail(SAGE_EINVAL, "out: base pointer and strides must be 8-byte aligned");
+  const bool packed = cu_seqlens_q != nullptr;
+  if (packed && (!cu_seqlens_k || !plan)) return fail(SAGE_EINVAL, "packed mode needs cu_seqlens_k and plan");
+  if (packed && B > 32767) return fail(SAGE_EINVAL, "too many sequences");
+  AttnConfig cfg = attn_config(D, pv_mode, packed);
+  const int BM = cfg.nw * 32;
+  AttnArgs a;
+  memset(&a, 0, sizeof(a));
+  a.q = q; a.k = k; a.vp = (const uint8_t*)v_panels; a.qs = q_scale; a.ks = k_scale; a.vs = v_scale;
+  a.out = out; a.lse = lse;
+  a.B = B; a.Hq = Hq; a.Hkv = Hkv; a.Sq = Sq; a.Skv = Skv;
+  a.q_sb = q_sb; a.q_sh = q_sh; a.q_sn = q_sn; a.k_sb = k_sb; a.k_sh = k_sh; a.k_sn = k_sn;
+  a.o_sb = o_sb; a.o_sh = o_sh; a.o_sn = o_sn;
+  a.blkq = blkq; a.blkk = blkk; a.out_bf16 = out_dtype == SAGE_DT_BF16;
+  a.nqt = (Sq + BM - 1) / BM;
+  int64_t grid;
+  if (packed) {
+    SagePlanLayout L = plan_layout(B, total_q);
+    a.cu_q = cu_seqlens_q; a.cu_k = cu_seqlens_k;
+    a.cu_qblk = plan + L.cu_qblk; a.cu_kblk = plan + L.cu_kblk; a.cu_panel = plan + L.cu_panel;
+    a.ntiles = plan + L.ntiles; a.tiles = plan + L.tiles;
+    a.qs_sh = q_scale_sh; a.ks_sh = k_scale_sh; a.panel_sh = panel_sh; a.total_q = total_q;
+    grid = ((int64_t)total_q / BM + B) * Hq;  // upper bound on tiles; surplus workgroups exit at once
+  } else {
+    grid = (int64_t)a.nqt * B * Hq;
+  }
+  if (grid > 0x7fffffff) return fail(SAGE_EINVAL, "too many tiles for one launch");
+  hipError_t e = launch_attn(a, D, pv_mode, is_causal != 0, (int)grid, (hipStream_t)stream);
+  if (e != hipSuccess) return hip_fail(e, "sage_attn_fwd");
+  return SAGE_OK;
+}
+
+// ---- one-call pipeline --------------------------------------------------------------------
+namespace {
+struct E2EWorkspace {
+  size_t q_i8, k_i8, q_scale, k_scale, km, v_scale, panels, stat, plan, total;
+  int64_t qs_sh, ks_sh, panel_sh;
+};
+E2EWorkspace e2e_layout(int B, int Hq, int Hkv, int Sq, int Skv, int D, int blkq, int blkk, int pv, int total_q, int total_k,
+                        int varlen) {
+  E2EWorkspace w;
+  size_t off = 0;
+  size_t nq = varlen ? (size_t)total_q * Hq * D : (size_t)B * Hq * Sq * D;
+  size_t nk = varlen ? (size_t)total_k * Hkv * D : (size_t)B * Hkv * Skv * D;
+  w.q_i8 = off; off += align_up(nq);
+  w.k_i8 = off; off += align_up(nk);
+  if (varlen) {
+    w.qs_sh = total_q / blkq + B; w.ks_sh = total_k / blkk + B; w.panel_sh = total_k / SAGE_PANEL_ROWS + B;
+    w.q_scale = off; off += align_up((size_t)Hq * w.qs_sh * 4);
+    w.k_scale = off; off += align_up((size_t)Hkv * w.ks_sh * 4);
+  } else {
+    w.qs_sh = w.ks_sh = w.panel_sh = 0;
+    w.q_scale = off; off += align_up((size_t)B * Hq * ((Sq + blkq - 1) / blkq) * 4);
+    w.k_scale = off; off += align_up((size_t)B * Hkv * ((Skv + blkk - 1) / blkk) * 4);
+  }
+  w.km = off; off += align_up((size_t)B * Hkv * D * 2);
+  w.v_scale = off; off += align_up((size_t)B * Hkv * D * 4);
+  size_t pbytes = varlen ? (size_t)Hkv * w.panel_sh * SAGE_PANEL_ROWS * D * (pv ? 1 : 2) : sage_v_panel_bytes(B, Hkv, Skv, D, pv);
+  w.panels = off; off += align_up(pbytes);
+  size_t stat = sage_k_mean_workspace_bytes(B, Hkv, Skv, D);
+  size_t stat2 = sage_prep_v_workspace_bytes(B, Hkv, Skv, D, pv);
+  w.stat = off; off += align_up(stat > stat2 ? stat : stat2);
+  w.plan = off; off += varlen ? align_up(sage_varlen_plan_ints(B, total_q) * 4) : 0;
+  w.total = off;
+  return w;
+}
+}  // namespace
+
+size_t sage_sageattn_workspace_bytes(int B, int Hq, int Hkv, int Sq, int Skv, int D, int blkq, int blkk, int pv_mode,
+                                     int total_q, int total_k, int varlen) {
+  if (blkq <= 0 || blkk <= 0) return 0;
+  return e2e_layout(B, Hq, Hkv, Sq, Skv, D, blkq, blkk, pv_mode, total_q, total_k, varlen).total;
+}
+
+int sage_sageattn(const void* q, const void* k, const void* v, void* out, float* lse, void* workspace, size_t workspace_bytes,
+                  int B, int Hq, int Hkv, int Sq, int Skv, int D, int64_t q_sb, int64_t q_sh, int64_t q_sn, int64_t k_sb,
+                  int64_t k_sh, int64_t k_sn, int64_t v_sb, int64_t v_sh, int64_t v_sn, int64_t o_sb, int64_t o_sh,
+                  int64_t o_sn, int dtype, int blkq, int blkk, double sm_scale, int is_causal, int smooth_k, int pv_mode,
+                  const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k, int total_q, int total_k, sage_stream_t stream) {
+  if (int rc = check_common(B, Hq, Sq, D, dtype)) return rc;
+  if (Hkv <= 0 || Hq % Hkv) return fail(SAGE_EINVAL, "query heads (%d) must be divisible by KV heads (%d)", Hq, Hkv);
+  if (blkq % 32 || blkk % 32 || blkq <= 0 || blkk <= 0 || blkq > 128 || blkk > 128)
+    return fail(SAGE_ENOTIMPL, "scale blocks must be multiples of 32 up to 128 (got %d/%d)", blkq, blkk);
+  if (pv_mode != SAGE_PV_FP16 && pv_mode != SAGE_PV_FP8) return fail(SAGE_EINVAL, "pv_mode %d unknown", pv_mode);
+  const int varlen = cu_seqlens_q != nullptr;
+  if (varlen && !cu_seqlens_k) return fail(SAGE_EINVAL, "packed mode needs cu_seqlens_k");
+  if (B == 0 || Hq == 0 || Sq == 0) return SAGE_OK;
+  if (!workspace) return fail(SAGE_EWORKSPACE, "null workspace");
+  E2EWorkspace w = e2e_layout(B, Hq, Hkv, Sq, Skv, D, blkq, blkk, pv_mode, total_q, total_k, varlen);
+  if (workspace_bytes < w.total) return fail(SAGE_EWORKSPACE, "workspace too small: %zu < %zu", workspace_bytes, w.total);
+  if (reinterpret_cast<uintptr_t>(workspace) % 256) return fail(SAGE_EINVAL, "workspace must be 256-byte aligned");
+  uint8_t* ws = (uint8_t*)workspace;
+  int8_t* q_i8 = (int8_t*)(ws + w.q_i8);
+  int8_t* k_i8 = (int8_t*)(ws + w.k_i8);
+  float* q_scale = (float*)(ws + w.q_scale);
+  float* k_scale = (float*)(ws + w.k_scale);
+  void* km = ws + w.km;
+  float* v_scale = (float*)(ws + w.v_scale);
+  void* panels = ws + w.panels;
+  void* stat = ws + w.stat;
+  int32_t* plan = varlen ? (int32_t*)(ws + w.plan) : nullptr;
+  const size_t stat_bytes = w.plan - w.stat;
+  // the int8 copies are dense in the caller's layout order: reuse the input strides scaled to D
+  // (HND/NHD/packed inputs are dense, so their element strides are valid for an int8 tensor too)
+  const int32_t *cu_qblk = nullptr, *cu_kblk = nullptr, *cu_panel = nullptr;
+  if (varlen) {
+    int rc = sage_varlen_plan(cu_seqlens_q, cu_seqlens_k, B, total_q, blkq, blkk, is_causal, plan,
+                              sage_varlen_plan_ints(B, total_q), stream);
+    if (rc) return rc;
+    SagePlanLayout L = plan_layout(B, total_q);
+    cu_qblk = plan + L.cu_qblk; cu_kblk = plan + L.cu_kblk; cu_panel = plan + L.cu_panel;
+  }
+  int rc;
+  if (smooth_k) {
+    rc = sage_k_mean(k, km, stat, stat_bytes, B, Hkv, Skv, D, k_sb, k_sh, k_sn, dtype, cu_seqlens_k, stream);
+    if (rc) return rc;
+  }
+  rc = sage_quant_int8(k, k_i8, k_scale, smooth_k ? km : nullptr, B, Hkv, Skv, D, k_sb, k_sh, k_sn, k_sb, k_sh, k_sn,
+                       (int64_t)Hkv * D, D, blkk, 1.0f, dtype, cu_seqlens_k, cu_kblk, w.ks_sh, stream);
+  if (rc) return rc;
+  rc = sage_quant_int8(q, q_i8, q_scale, nullptr, B, Hq, Sq, D, q_sb, q_sh, q_sn, q_sb, q_sh, q_sn, 0, 0, blkq,
+                       (float)((sm_scale > 0 ? sm_scale : 1.0 / sqrt((double)D)) * 1.44269504), dtype, cu_seqlens_q, cu_qblk, w.qs_sh, stream);
+  if (rc) return rc;
+  rc = sage_prep_v(v, panels, v_scale, stat, stat_bytes, B, Hkv, Skv, D, v_sb, v_sh, v_sn, dtype, pv_mode, cu_seqlens_k,
+                   cu_panel, w.panel_sh, stream);
+  if (rc) return rc;
+  return sage_attn_fwd(q_i8, k_i8, panels, q_scale, k_scale, pv_mode == SAGE_PV_FP8 ? v_scale : nullptr, out, lse, B, Hq, Hkv,
+                       Sq, Skv, D, q_sb, q_sh, q_sn, k_sb, k_sh, k_sn, o_sb, o_sh, o_sn, blkq, blkk, is_causal, pv_mode, dtype,
+                       cu_seqlens_q, cu_seqlens_k, plan, total_q, w.qs_sh, w.ks_sh, w.panel_sh, stream);
+}
+
+}  // extern "C"

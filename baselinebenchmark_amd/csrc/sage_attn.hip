@@ -1,0 +1,443 @@
+// Fused SageAttention forward kernel for gfx950 (MI355X).
+//
+// Replaces _attention_kernel of backends/_hygon/ops/sageattention/sageattention_triton.py:45-129
+// (INT8 Q.K^T, fp32 base-2 online softmax, P.V with fp32 accumulation, O/l epilogue, LSE2) and adds
+// causal block skipping, tail masking, FP8 P.V and packed variable-length batches.
+//
+// Mapping to the hardware
+//   * A workgroup of NW wavefronts owns a q-tile of BM = 32*NW rows of one (batch, q-head); each
+//     wavefront owns 32 query rows for the whole KV loop.
+//   * Everything is computed TRANSPOSED so that a query row lives in one lane column:
+//       S^T[n, m] = K[n, :] . Q[m, :]      v_mfma_i32_32x32x32_i8      A = K tile (LDS), B = Q (regs)
+//       O^T[d, m] = V^T[d, n] . P^T[n, m]   v_mfma_f32_32x32x64_f8f6f4  A = V panel (LDS), B = P (regs)
+//                                       or  v_mfma_f32_32x32x16_f16
+//     In the 32x32 accumulator layout lane (m = lane%32, h = lane/32) holds column m, rows
+//     8*(r/4) + 4*h + r%4.  So row max / row sum of query row m are in-lane reductions plus ONE
+//     exchange with lane m+32 (v_permlane32_swap), the probabilities are already laid out as the
+//     B operand of the second MFMA (V panels are pre-permuted to match, see sage_common.h), and the
+//     running rescale / final 1/l multiply the lane's own accumulators.
+//   * The INT32 accumulators start from the bit pattern of 1.5*2^23, so reading them as floats gives
+//     12582912 + dot exactly: the int->float conversion is folded into the one FMA that applies
+//     q_scale*k_scale and subtracts the running maximum.
+//   * The running maximum is only moved when it grows by more than kTau (lazy rescale); P is stored
+//     with a static 2^kPShift so that fp8's range [2^-9, 448] is used.
+//   * K/V tiles go global -> registers -> LDS, double buffered, one barrier per KV tile.
+#include "sage_launch.h"
+
+namespace sage {
+
+
+constexpr float kBiasF = 12582912.0f;     // 1.5 * 2^23
+constexpr int kBiasBits = 0x4B400000;     // its bit pattern; int accumulators start here
+constexpr float kNegInf = -__builtin_inff();
+constexpr float kMInit = -1.0e30f;
+
+template <int PV> struct PCfg;
+template <> struct PCfg<1> { static constexpr float tau = 3.0f, pshift = 5.0f; };   // fp8: p*32 <= 256 < 448
+template <> struct PCfg<0> { static constexpr float tau = 8.0f, pshift = 0.0f; };   // fp16: p <= 256
+
+// NOTE: __builtin_bit_cast applied directly to an element of an ext_vector_type value reads element
+// 0 whatever the index (clang miscompiles the element lvalue), so vector elements are always passed
+// BY VALUE through these two helpers.
+__device__ inline float as_f(int v) { return __builtin_bit_cast(float, v); }
+__device__ inline int as_i(float v) { return __builtin_bit_cast(int, v); }
+
+// Exchange between lane l and lane l^32 (the two lanes that share a query row).
+// v_permlane32_swap swaps the upper half of its first operand with the lower half of its second, so
+// with both operands holding x every lane ends up with {x[l%32], x[l%32 + 32]}.
+__device__ inline void xchg32(float x, float& lo, float& hi) {
+  auto r = __builtin_amdgcn_permlane32_swap(as_i(x), as_i(x), false, false);
+  int r0 = r[0], r1 = r[1];
+  lo = as_f(r0);
+  hi = as_f(r1);
+}
+__device__ inline float xchg32_max(float x) {
+  float lo, hi;
+  xchg32(x, lo, hi);
+  return fmaxf(lo, hi);
+}
+__device__ inline float xchg32_sum(float x) {
+  float lo, hi;
+  xchg32(x, lo, hi);
+  return lo + hi;
+}
+
+// 16-byte-chunk swizzle of a K row in LDS: consecutive rows read the same logical chunk from
+// different bank groups (64 banks x 4 bytes = 256 bytes per bank row).
+template <int D>
+__device__ inline int kswz(int n) {
+  constexpr int CPR = D / 16, RPB = 256 / D;
+  return (n / RPB) % CPR;
+}
+
+template <int D, int NW, int BN, int PV, bool CAUSAL>
+__global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
+  constexpr int BM = NW * 32;
+  constexpr int NTHR = NW * 64;
+  constexpr int KS = D / 32;   // contraction steps of S^T
+  constexpr int NT = BN / 32;  // 32-row tiles of S^T
+  constexpr int DTN = D / 32;  // 32-row tiles of O^T
+  constexpr int VESZ = PV ? 1 : 2;
+  constexpr int KBYTES = BN * D, VBYTES = BN * D * VESZ, STAGE = KBYTES + VBYTES;
+  constexpr int KCHUNKS = KBYTES / 16, VCHUNKS = VBYTES / 16;
+  constexpr int KCH = (KCHUNKS + NTHR - 1) / NTHR, VCH = (VCHUNKS + NTHR - 1) / NTHR;
+  constexpr int PANEL_BYTES = kPanelRows * D * VESZ;
+  constexpr int CPR = D / 16;
+  constexpr float TAU = PCfg<PV>::tau, PSHIFT = PCfg<PV>::pshift;
+
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int m = lane & 31, h = lane >> 5;
+
+  // ---- which tile am I: heaviest q-tiles first; q-heads sharing a KV head on one XCD ----
+  const bool packed = a.cu_q != nullptr;
+  const int G = a.Hq / a.Hkv;
+  int rank, s, NG;
+  if (packed) { rank = blockIdx.x / a.Hq; s = blockIdx.x % a.Hq; NG = a.Hkv; }
+  else { int U = a.B * a.Hq; rank = blockIdx.x / U; s = blockIdx.x % U; NG = a.B * a.Hkv; }
+  int gi, g;
+  if ((NG & 7) == 0) { int x = s & 7, y = s >> 3; gi = x + 8 * (y / G); g = y % G; }
+  else { gi = s / G; g = s % G; }
+  int b, kvh, qt, Lq, Lk;
+  int64_t qoff, koff, ooff, lseoff;
+  const float *qsp, *ksp;
+  const uint8_t* vbase;
+  int nkblk;
+  if (packed) {
+    if (rank >= a.ntiles[0]) return;
+    int t = a.tiles[rank];
+    b = t >> 16; qt = t & 0xffff; kvh = gi;
+    int q0 = a.cu_q[b], k0 = a.cu_k[b];
+    Lq = a.cu_q[b + 1] - q0; Lk = a.cu_k[b + 1] - k0;
+    int hq = kvh * G + g;
+    qoff = (int64_t)q0 * a.q_sn + (int64_t)hq * a.q_sh;
+    ooff = (int64_t)q0 * a.o_sn + (int64_t)hq * a.o_sh;
+    koff = (int64_t)k0 * a.k_sn + (int64_t)kvh * a.k_sh;
+    lseoff = (int64_t)hq * a.total_q + q0;
+    qsp = a.qs + (int64_t)hq * a.qs_sh + a.cu_qblk[b];
+    ksp = a.ks + (int64_t)kvh * a.ks_sh + a.cu_kblk[b];
+    vbase = a.vp + ((int64_t)kvh * a.panel_sh + a.cu_panel[b]) * PANEL_BYTES;
+  } else {
+    b = gi / a.Hkv; kvh = gi % a.Hkv;
+    qt = CAUSAL ? a.nqt - 1 - rank : rank;
+    Lq = a.Sq; Lk = a.Skv;
+    int hq = kvh * G + g;
+    qoff = (int64_t)b * a.q_sb + (int64_t)hq * a.q_sh;
+    ooff = (int64_t)b * a.o_sb + (int64_t)hq * a.o_sh;
+    koff = (int64_t)b * a.k_sb + (int64_t)kvh * a.k_sh;
+    lseoff = ((int64_t)b * a.Hq + hq) * a.Sq;
+    qsp = a.qs + ((int64_t)b * a.Hq + hq) * ((Lq + a.blkq - 1) / a.blkq);
+    ksp = a.ks + ((int64_t)b * a.Hkv + kvh) * ((Lk + a.blkk - 1) / a.blkk);
+    vbase = a.vp + ((int64_t)b * a.Hkv + kvh) * ((Lk + kPanelRows - 1) / kPanelRows) * PANEL_BYTES;
+  }
+  nkblk = (Lk + a.blkk - 1) / a.blkk;
+
+  const int row0 = qt * BM + w * 32;   // first query row of this wavefront
+  const int my_row = row0 + m;
+  const int kv_end = CAUSAL ? min(Lk, qt * BM + BM) : Lk;
+  const int ntiles = (kv_end + BN - 1) / BN;
+  const int wave_end = (row0 < Lq) ? (CAUSAL ? min(Lk, row0 + 32) : Lk) : 0;
+  const int wave_ntiles = (wave_end + BN - 1) / BN;
+
+  // ---- Q operand: lane (m, h) holds bytes 32*ks + 16*h .. +15 of its row for every ks ----
+  v4i qreg[KS];
+  {
+    const int8_t* qp = a.q + qoff + (int64_t)min(my_row, Lq - 1) * a.q_sn + 16 * h;
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) qreg[ks] = *reinterpret_cast<const v4i*>(qp + 32 * ks);
+  }
+  const float qscale = qsp[min(row0, Lq - 1) / a.blkq];
+
+  v16i bias;
+#pragma unroll
+  for (int i = 0; i < 16; i++) bias[i] = kBiasBits;
+  asm volatile("" : "+v"(bias));  // keep it in registers: it is the C operand of every first MFMA
+
+  v16f o[DTN];
+#pragma unroll
+  for (int dt = 0; dt < DTN; dt++)
+#pragma unroll
+    for (int i = 0; i < 16; i++) o[dt][i] = 0.f;
+  float m_used = kMInit, lsum = 0.f;
+
+  // ---- cooperative tile loads: global -> registers, registers -> LDS ----
+  v4i kst[KCH], vst[VCH];
+  auto load_tile = [&](int j) {
+    const int n0 = j * BN;
+#pragma unroll
+    for (int i = 0; i < KCH; i++) {
+      int c = i * NTHR + tid, n = c / CPR, cc = c % CPR;
+      int row = min(n0 + n, Lk - 1);
+      if (KCHUNKS % NTHR == 0 || c < KCHUNKS)
+        kst[i] = *reinterpret_cast<const v4i*>(a.k + koff + (int64_t)row * a.k_sn + 16 * cc);
+    }
+    const uint8_t* vsrc = vbase + (int64_t)n0 * D * VESZ;
+#pragma unroll
+    for (int i = 0; i < VCH; i++)
+      if (VCHUNKS % NTHR == 0 || i * NTHR + tid < VCHUNKS)
+        vst[i] = *reinterpret_cast<const v4i*>(vsrc + (int64_t)(i * NTHR + tid) * 16);
+  };
+  auto store_tile = [&](uint8_t* stage) {
+#pragma unroll
+    for (int i = 0; i < KCH; i++) {
+      int c = i * NTHR + tid, n = c / CPR, cc = c % CPR;
+      if (KCHUNKS % NTHR == 0 || c < KCHUNKS)
+        *reinterpret_cast<v4i*>(stage + n * D + 16 * (cc ^ kswz<D>(n))) = kst[i];
+    }
+#pragma unroll
+    for (int i = 0; i < VCH; i++)
+      if (VCHUNKS % NTHR == 0 || i * NTHR + tid < VCHUNKS)
+        *reinterpret_cast<v4i*>(stage + KBYTES + (i * NTHR + tid) * 16) = vst[i];
+  };
+
+  auto compute = [&](const uint8_t* stage, int j) {
+    const int n0 = j * BN;
+    const uint8_t* kbuf = stage;
+    const uint8_t* vbuf = stage + KBYTES;
+    // ---- S^T = K . Q^T (int8 -> int32 on the biased accumulators) ----
+    v16i acc[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; nt++) {
+      const int n = 32 * nt + m;
+      const uint8_t* rowp = kbuf + n * D;
+      const int sw = kswz<D>(n);
+#pragma unroll
+      for (int ks = 0; ks < KS; ks++) {
+        v4i ka = *reinterpret_cast<const v4i*>(rowp + 16 * ((2 * ks + h) ^ sw));
+        acc[nt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ka, qreg[ks], ks == 0 ? bias : acc[nt], 0, 0, 0);
+      }
+    }
+    float sc[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; nt++) sc[nt] = qscale * ksp[min((n0 + 32 * nt) / a.blkk, nkblk - 1)];
+
+    // ---- masking: only tiles that cross the diagonal or the end of the sequence ----
+    const bool need_mask = (CAUSAL && (n0 + BN - 1 > row0)) || (n0 + BN > Lk);
+    if (need_mask) {
+      const int lim = (CAUSAL ? min(my_row, Lk - 1) : Lk - 1) - n0 - 4 * h;
+#pragma unroll
+      for (int nt = 0; nt < NT; nt++)
+#pragma unroll
+        for (int r = 0; r < 16; r++)
+          if (32 * nt + 8 * (r / 4) + (r % 4) > lim) acc[nt][r] = as_i(kNegInf);
+    }
+
+    // ---- row maximum of this tile, in score units ----
+    float mloc = kNegInf;
+#pragma unroll
+    for (int nt = 0; nt < NT; nt++) {
+      float mx = as_f(acc[nt][0]);
+#pragma unroll
+      for (int r = 1; r < 16; r++) mx = fmaxf(mx, as_f(acc[nt][r]));
+      mloc = fmaxf(mloc, __builtin_fmaf(mx, sc[nt], -kBiasF * sc[nt]));
+    }
+    mloc = xchg32_max(mloc);
+
+    // ---- lazy rescale: move the reference maximum only when it grew by more than TAU ----
+    if (__builtin_amdgcn_ballot_w64(mloc > m_used + TAU) != 0) {
+      const float m_new = fmaxf(m_used, mloc);
+      const float alpha = __builtin_amdgcn_exp2f(m_used - m_new);
+      lsum *= alpha;
+#pragma unroll
+      for (int dt = 0; dt < DTN; dt++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) o[dt][i] *= alpha;
+      m_used = m_new;
+    }
+
+    // ---- P = exp2(S - m) * 2^PSHIFT, packed straight into the B operand of the second MFMA ----
+    if constexpr (PV == 1) {
+      v4i pk[NT];
+#pragma unroll
+      for (int nt = 0; nt < NT; nt++) {
+        const float c = __builtin_fmaf(-kBiasF, sc[nt], PSHIFT - m_used);
+        float p[16];
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          p[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(as_f(acc[nt][r]), sc[nt], c));
+          lsum += p[r];
+        }
+#pragma unroll
+        for (int q4 = 0; q4 < 4; q4++) {
+          int d0 = __builtin_amdgcn_cvt_pk_fp8_f32(p[4 * q4], p[4 * q4 + 1], 0, false);
+          pk[nt][q4] = __builtin_amdgcn_cvt_pk_fp8_f32(p[4 * q4 + 2], p[4 * q4 + 3], d0, true);
+        }
+      }
+      // ---- O^T += V^T . P^T ----
+#pragma unroll
+      for (int kk = 0; kk < BN / 64; kk++) {
+        v8i pb;
+#pragma unroll
+        for (int i = 0; i < 4; i++) { pb[i] = pk[2 * kk][i]; pb[4 + i] = pk[2 * kk + 1][i]; }
+#pragma unroll
+        for (int dt = 0; dt < DTN; dt++) {
+          const uint8_t* vp0 = vbuf + (((kk * DTN + dt) * 2) * 64 + lane) * 16;
+          v4i lo = *reinterpret_cast<const v4i*>(vp0);
+          v4i hi = *reinterpret_cast<const v4i*>(vp0 + 64 * 16);
+          v8i va = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+          o[dt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(va, pb, o[dt], 0, 0, 0, 0, 0, 0);
+        }
+      }
+    } else {
+      v8h ph[NT][2];
+#pragma unroll
+      for (int nt = 0; nt < NT; nt++) {
+        const float c = __builtin_fmaf(-kBiasF, sc[nt], PSHIFT - m_used);
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          float p = __builtin_amdgcn_exp2f(__builtin_fmaf(as_f(acc[nt][r]), sc[nt], c));
+          lsum += p;
+          ph[nt][r >> 3][r & 7] = (_Float16)p;
+        }
+      }
+#pragma unroll
+      for (int k16 = 0; k16 < BN / 16; k16++) {
+#pragma unroll
+        for (int dt = 0; dt < DTN; dt++) {
+          v8h va = *reinterpret_cast<const v8h*>(vbuf + ((k16 * DTN + dt) * 64 + lane) * 16);
+          o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va, ph[k16 >> 1][k16 & 1], o[dt], 0, 0, 0);
+        }
+      }
+    }
+  };
+
+  // ---- main loop over KV tiles ----
+  if (ntiles > 0) {
+    load_tile(0);
+    store_tile(smem);
+    __syncthreads();
+    for (int j = 0; j < ntiles; j++) {
+      uint8_t* cur = smem + (j & 1) * STAGE;
+      uint8_t* nxt = smem + ((j + 1) & 1) * STAGE;
+      if (j + 1 < ntiles) load_tile(j + 1);
+      if (j < wave_ntiles) compute(cur, j);
+      if (j + 1 < ntiles) store_tile(nxt);
+      __syncthreads();
+    }
+  }
+
+  // ---- epilogue: O = O^T / l (* v_scale), LSE2 = m + log2(l) ----
+  lsum = xchg32_sum(lsum);
+  const float inv = lsum > 0.f ? 1.0f / lsum : 0.f;
+  if (my_row < Lq) {
+    if (a.lse && h == 0) a.lse[lseoff + my_row] = lsum > 0.f ? m_used + __builtin_amdgcn_logf(lsum) - PSHIFT : kNegInf;
+    const int64_t orow = ooff + (int64_t)my_row * a.o_sn;
+#pragma unroll
+    for (int dt = 0; dt < DTN; dt++) {
+#pragma unroll
+      for (int q4 = 0; q4 < 4; q4++) {
+        const int d = 32 * dt + 8 * q4 + 4 * h;
+        float f[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          f[i] = o[dt][4 * q4 + i] * inv;
+          if constexpr (PV == 1) f[i] *= a.vs[((int64_t)b * a.Hkv + kvh) * D + d + i];
+        }
+        u16 hv[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) hv[i] = a.out_bf16 ? f32_to_bf16(f[i]) : f32_to_f16(f[i]);
+        uint2 pkd = make_uint2((uint32_t)hv[0] | ((uint32_t)hv[1] << 16), (uint32_t)hv[2] | ((uint32_t)hv[3] << 16));
+        *reinterpret_cast<uint2*>(reinterpret_cast<u16*>(a.out) + orow + d) = pkd;
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Variable-length plan: block offsets per sequence and the cost-ordered tile list.
+// One workgroup; sequences are few (tens to thousands), tiles up to total_q/128 + nseq.
+// ---------------------------------------------------------------------------------------------
+constexpr int kCostBins = 2048;
+
+__global__ void __launch_bounds__(1024) varlen_plan_kernel(const int32_t* cu_q, const int32_t* cu_k, int nseq, int total_q,
+                                                           int blkq, int blkk, int bm, int bn, int causal, int32_t* plan) {
+  const SagePlanLayout L = plan_layout(nseq, total_q);
+  int32_t* cu_qblk = plan + L.cu_qblk;
+  int32_t* cu_kblk = plan + L.cu_kblk;
+  int32_t* cu_panel = plan + L.cu_panel;
+  int32_t* tiles = plan + L.tiles;
+  __shared__ int hist[kCostBins];
+  __shared__ int start[kCostBins];
+  const int tid = threadIdx.x;
+  for (int i = tid; i < kCostBins; i += blockDim.x) hist[i] = 0;
+  if (tid == 0) {
+    int aq = 0, ak = 0, ap = 0;
+    for (int i = 0; i < nseq; i++) {
+      cu_qblk[i] = aq; cu_kblk[i] = ak; cu_panel[i] = ap;
+      int lq = cu_q[i + 1] - cu_q[i], lk = cu_k[i + 1] - cu_k[i];
+      aq += (lq + blkq - 1) / blkq; ak += (lk + blkk - 1) / blkk; ap += (lk + kPanelRows - 1) / kPanelRows;
+    }
+    cu_qblk[nseq] = aq; cu_kblk[nseq] = ak; cu_panel[nseq] = ap;
+  }
+  __syncthreads();
+  auto cost_of = [&](int lq, int lk, int qt) {
+    int kv_end = causal ? min(lk, (qt + 1) * bm) : lk;
+    int c = (kv_end + bn - 1) / bn;
+    return min(c, kCostBins - 1);
+  };
+  // pass 1: histogram of tile costs
+  for (int i = 0; i < nseq; i++) {
+    int lq = cu_q[i + 1] - cu_q[i], lk = cu_k[i + 1] - cu_k[i];
+    int nqt = (lq + bm - 1) / bm;
+    for (int qt = tid; qt < nqt; qt += blockDim.x) atomicAdd(&hist[cost_of(lq, lk, qt)], 1);
+  }
+  __syncthreads();
+  if (tid == 0) {
+    int acc = 0;
+    for (int c = kCostBins - 1; c >= 0; c--) { start[c] = acc; acc += hist[c]; }
+    plan[L.ntiles] = acc;
+  }
+  __syncthreads();
+  // pass 2: place tiles, most expensive bins first
+  for (int i = 0; i < nseq; i++) {
+    int lq = cu_q[i + 1] - cu_q[i], lk = cu_k[i + 1] - cu_k[i];
+    int nqt = (lq + bm - 1) / bm;
+    for (int qt = tid; qt < nqt; qt += blockDim.x) {
+      int pos = atomicAdd(&start[cost_of(lq, lk, qt)], 1);
+      tiles[pos] = (i << 16) | qt;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Launchers
+// ---------------------------------------------------------------------------------------------
+AttnConfig attn_config(int D, int pv, bool packed) {
+  (void)D; (void)packed;
+  AttnConfig c;
+  c.nw = 8;
+  c.bn = pv ? 128 : 64;
+  return c;
+}
+
+template <int D, int NW, int BN, int PV, bool CAUSAL>
+static hipError_t launch_one(const AttnArgs& a, int grid, hipStream_t st) {
+  constexpr int VESZ = PV ? 1 : 2;
+  constexpr int smem = 2 * (BN * D + BN * D * VESZ);
+  auto kern = attn_kernel<D, NW, BN, PV, CAUSAL>;
+  static bool attr_done = false;
+  if (!attr_done) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) return e;
+    attr_done = true;
+  }
+  kern<<<dim3(grid), dim3(NW * 64), smem, st>>>(a);
+  return hipGetLastError();
+}
+
+hipError_t launch_attn(const AttnArgs& a, int D, int pv, bool causal, int grid, hipStream_t st) {
+  if (grid == 0) return hipSuccess;
+#define SAGE_ATTN(DD, PVV, BNN) (causal ? launch_one<DD, 8, BNN, PVV, true>(a, grid, st) : launch_one<DD, 8, BNN, PVV, false>(a, grid, st))
+  if (D == 128) return pv ? SAGE_ATTN(128, 1, 128) : SAGE_ATTN(128, 0, 64);
+  return pv ? SAGE_ATTN(64, 1, 128) : SAGE_ATTN(64, 0, 64);
+#undef SAGE_ATTN
+}
+
+hipError_t launch_varlen_plan(const int32_t* cu_q, const int32_t* cu_k, int nseq, int total_q, int blkq, int blkk, int bm,
+                              int bn, int causal, int32_t* plan, hipStream_t st) {
+  varlen_plan_kernel<<<1, 1024, 0, st>>>(cu_q, cu_k, nseq, total_q, blkq, blkk, bm, bn, causal, plan);
+  return hipGetLastError();
+}
+
+}  // namespace sage

@@ -1,0 +1,80 @@
+// Host-side launcher declarations shared between the kernel translation units and the C ABI.
+#pragma once
+#include "sage_common.h"
+
+namespace sage {
+
+struct QuantArgs {
+  const u16* x;
+  int8_t* out;
+  float* scale;
+  const u16* km;
+  int B, H, L, D;
+  int64_t x_sb, x_sh, x_sn, o_sb, o_sh, o_sn, km_sb, km_sh;
+  int blk;
+  float mult;
+  const int32_t* cu_seqlens;
+  const int32_t* cu_blocks;
+  int64_t scale_sh;
+};
+
+struct ColStatArgs {
+  const u16* x;
+  void* partial;  // double or float [B*H*nchunk*D]
+  int B, H, L, D;
+  int64_t x_sb, x_sh, x_sn;
+  int nchunk;
+  const int32_t* cu_seqlens;
+};
+
+struct PrepVArgs {
+  const u16* v;
+  uint8_t* panels;
+  const float* vscale;  // [B*H*D] (fp8) or null
+  int B, H, L, D;
+  int64_t v_sb, v_sh, v_sn;
+  const int32_t* cu_seqlens;
+  const int32_t* cu_panels;
+  int64_t panel_sh;
+};
+
+struct AttnArgs {
+  const int8_t* q;
+  const int8_t* k;
+  const uint8_t* vp;
+  const float* qs;
+  const float* ks;
+  const float* vs;
+  void* out;
+  float* lse;
+  int B, Hq, Hkv, Sq, Skv;
+  int64_t q_sb, q_sh, q_sn, k_sb, k_sh, k_sn, o_sb, o_sh, o_sn;
+  int blkq, blkk;
+  int out_bf16;
+  int nqt;  // q-tiles per sequence (fixed-length mode)
+  // packed mode (cu_q != nullptr)
+  const int32_t* cu_q;
+  const int32_t* cu_k;
+  const int32_t* cu_qblk;
+  const int32_t* cu_kblk;
+  const int32_t* cu_panel;
+  const int32_t* ntiles;
+  const int32_t* tiles;
+  int64_t qs_sh, ks_sh, panel_sh;
+  int total_q;
+};
+
+struct AttnConfig { int nw, bn; };
+
+hipError_t launch_quant_int8(const QuantArgs& a, int dtype, int max_blocks, hipStream_t st);
+int colstat_chunks(int L);
+hipError_t launch_k_mean(const ColStatArgs& a, int dtype, void* km, hipStream_t st);
+hipError_t launch_v_scale(const ColStatArgs& a, int dtype, float* vscale, hipStream_t st);
+hipError_t launch_prep_v(const PrepVArgs& a, int dtype, int pv, int max_panels, hipStream_t st);
+
+AttnConfig attn_config(int D, int pv, bool packed);
+hipError_t launch_attn(const AttnArgs& a, int D, int pv, bool causal, int grid, hipStream_t st);
+hipError_t launch_varlen_plan(const int32_t* cu_q, const int32_t* cu_k, int nseq, int total_q, int blkq, int blkk, int bm,
+                              int bn, int causal, int32_t* plan, hipStream_t st);
+
+}  // namespace sage

@@ -1,0 +1,323 @@
+// Quantisers of the SageAttention forward path for gfx950 (MI355X):
+//   * per-block INT8 quantiser for Q and K (optional K-mean subtraction in the input dtype),
+//   * per-(batch, head, channel) column statistics over the sequence (K mean, V abs-max),
+//   * V preparation into MFMA-ready panels (fp16, or fp8-e4m3fn with per-channel scales).
+// All of them are streaming kernels bound by HBM bandwidth: 128-bit loads of 8 elements per
+// lane, statistics reduced with DPP inside the wavefront and through LDS across wavefronts.
+//
+// Arithmetic contract of the INT8 quantiser (bit-exact target): IEEE binary32 throughout,
+//   backends/_enflame/ops/sage_attention/quant_per_block.py:38-46  (+ :53-54 for k - km)
+//   backends/_hygon/ops/sageattention/sageattention_triton.py:35   (1e-12 floor)
+#include "sage_launch.h"
+
+#pragma clang fp contract(off)
+
+namespace sage {
+
+constexpr float kScaleFloor = 1.0e-12f;
+
+
+// Correctly rounded x / s for a wavefront-uniform divisor whose reciprocal r = RN(1/s) is given.
+// q0 = RN(x*r) is within 1 ulp of x/s; e = x - q0*s is exact in one FMA; RN(q0 + e*r) is then
+// the correctly rounded quotient (Markstein's correction step), provided s's significand is not
+// all ones and nothing under/overflows; the caller falls back to a true division otherwise.
+__device__ inline float div_by_uniform(float x, float s, float r) {
+  float q0 = x * r;
+  float e = __builtin_fmaf(-q0, s, x);
+  return __builtin_fmaf(e, r, q0);
+}
+
+// One workgroup (256 lanes) quantises one [blk, D] tile held entirely in registers:
+// pass 1 converts and reduces |x| to the tile maximum, pass 2 divides and rounds.
+template <int DT, int D>
+__global__ void __launch_bounds__(256) quant_int8_kernel(QuantArgs a) {
+  constexpr int TPR = D / 8;        // lanes per row (8 elements = 16 bytes each)
+  constexpr int RPP = 256 / TPR;    // rows per pass
+  constexpr int MAXP = 128 / RPP;   // passes for the largest tile (128 rows)
+  const int blkid = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const int tid = threadIdx.x;
+  const int tr = tid / TPR, tc = tid % TPR;
+
+  int L = a.L;
+  int64_t xbase, obase, sidx;
+  if (a.cu_seqlens) {
+    int s0 = a.cu_seqlens[b];
+    L = a.cu_seqlens[b + 1] - s0;
+    xbase = (int64_t)s0 * a.x_sn + (int64_t)h * a.x_sh;
+    obase = (int64_t)s0 * a.o_sn + (int64_t)h * a.o_sh;
+    sidx = (int64_t)h * a.scale_sh + a.cu_blocks[b] + blkid;
+  } else {
+    xbase = (int64_t)b * a.x_sb + (int64_t)h * a.x_sh;
+    obase = (int64_t)b * a.o_sb + (int64_t)h * a.o_sh;
+    sidx = ((int64_t)b * a.H + h) * ((L + a.blk - 1) / a.blk) + blkid;
+  }
+  const int n0 = blkid * a.blk;
+  if (n0 >= L) return;
+  const int rows = min(a.blk, L - n0);
+
+  float kmv[8];
+  const bool has_km = a.km != nullptr;
+  if (has_km) {
+    uint4 raw = *reinterpret_cast<const uint4*>(a.km + (int64_t)b * a.km_sb + (int64_t)h * a.km_sh + tc * 8);
+    const u16* p = reinterpret_cast<const u16*>(&raw);
+#pragma unroll
+    for (int i = 0; i < 8; i++) kmv[i] = to_f32<DT>(p[i]);
+  }
+
+  uint4 raw[MAXP];
+  float amax = 0.f;
+#pragma unroll
+  for (int p = 0; p < MAXP; p++) {
+    int r = p * RPP + tr;
+    raw[p] = make_uint4(0, 0, 0, 0);
+    if (r < rows) {
+      raw[p] = *reinterpret_cast<const uint4*>(a.x + xbase + (int64_t)(n0 + r) * a.x_sn + tc * 8);
+      const u16* e = reinterpret_cast<const u16*>(&raw[p]);
+#pragma unroll
+      for (int i = 0; i < 8; i++) {
+        float x = to_f32<DT>(e[i]);
+        if (has_km) x = to_f32<DT>(from_f32<DT>(x - kmv[i]));
+        x = x * a.mult;
+        amax = fmaxf(amax, fabsf(x));
+      }
+    }
+  }
+  __shared__ float wmax[4];
+  amax = wave_max(amax);
+  if ((tid & 63) == 0) wmax[tid >> 6] = amax;
+  __syncthreads();
+  amax = fmaxf(fmaxf(wmax[0], wmax[1]), fmaxf(wmax[2], wmax[3]));
+  const float scale = fmaxf(amax / 127.0f, kScaleFloor);
+  if (tid == 0) a.scale[sidx] = scale;
+
+  const float rcp = 1.0f / scale;
+  // The fast correction-step division needs: significand of scale not all ones, and scale, rcp
+  // and every quotient comfortably normal.  |quotient| <= 127.5, scale >= 1e-12.
+  const uint32_t sbits = __builtin_bit_cast(uint32_t, scale);
+  const bool fast = ((sbits & 0x7fffffu) != 0x7fffffu) && scale < 1.0e30f;
+
+#pragma unroll
+  for (int p = 0; p < MAXP; p++) {
+    int r = p * RPP + tr;
+    if (r < rows) {
+      const u16* e = reinterpret_cast<const u16*>(&raw[p]);
+      uint32_t packed[2] = {0, 0};
+#pragma unroll
+      for (int i = 0; i < 8; i++) {
+        float x = to_f32<DT>(e[i]);
+        if (has_km) x = to_f32<DT>(from_f32<DT>(x - kmv[i]));
+        x = x * a.mult;
+        float z;
+        if (fast) {
+          z = div_by_uniform(x, scale, rcp);
+          // tiny |x| could make the residual subnormal; its quotient is below 1e-13 in magnitude
+          // (scale >= 1e-12) and rounds to 0 whatever its sign
+          if (fabsf(x) < 1.0e-25f) z = 0.f;
+        } else {
+          z = x / scale;
+        }
+        z = (z >= 0.f) ? z + 0.5f : z - 0.5f;
+        int q = (int)z;  // truncation toward zero
+        packed[i >> 2] |= (uint32_t)(q & 0xff) << (8 * (i & 3));
+      }
+      *reinterpret_cast<uint2*>(a.out + obase + (int64_t)(n0 + r) * a.o_sn + tc * 8) = make_uint2(packed[0], packed[1]);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Column statistics over the sequence: MODE 0 = float64 sum (K mean), MODE 1 = fp32 abs-max (V).
+// Stage 1: one workgroup per (chunk of kChunkRows rows, head, batch) writes D partials.
+// Stage 2: one workgroup per (head, batch) combines the partials in chunk order.
+// ---------------------------------------------------------------------------------------------
+constexpr int kChunkRows = 512;
+
+
+template <int DT, int D, int MODE>
+__global__ void __launch_bounds__(256) colstat_partial_kernel(ColStatArgs a) {
+  using acc_t = typename std::conditional<MODE == 0, double, float>::type;
+  constexpr int TPR = D / 8, RPP = 256 / TPR;
+  const int chunk = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const int tid = threadIdx.x, tr = tid / TPR, tc = tid % TPR;
+  int L = a.L;
+  int64_t xbase;
+  if (a.cu_seqlens) {
+    int s0 = a.cu_seqlens[b];
+    L = a.cu_seqlens[b + 1] - s0;
+    xbase = (int64_t)s0 * a.x_sn + (int64_t)h * a.x_sh;
+  } else {
+    xbase = (int64_t)b * a.x_sb + (int64_t)h * a.x_sh;
+  }
+  const int n0 = chunk * kChunkRows;
+  if (n0 >= L) return;
+  const int n1 = min(L, n0 + kChunkRows);
+  acc_t acc[8];
+#pragma unroll
+  for (int i = 0; i < 8; i++) acc[i] = 0;
+  for (int n = n0 + tr; n < n1; n += RPP) {
+    uint4 raw = *reinterpret_cast<const uint4*>(a.x + xbase + (int64_t)n * a.x_sn + tc * 8);
+    const u16* e = reinterpret_cast<const u16*>(&raw);
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      float x = to_f32<DT>(e[i]);
+      if constexpr (MODE == 0) acc[i] += (double)x;
+      else acc[i] = fmaxf(acc[i], fabsf(x));
+    }
+  }
+  __shared__ acc_t red[RPP][D];
+#pragma unroll
+  for (int i = 0; i < 8; i++) red[tr][tc * 8 + i] = acc[i];
+  __syncthreads();
+  if (tid < D) {
+    acc_t t = red[0][tid];
+    for (int r = 1; r < RPP; r++) {
+      if constexpr (MODE == 0) t += red[r][tid];
+      else t = fmaxf(t, red[r][tid]);
+    }
+    reinterpret_cast<acc_t*>(a.partial)[(((int64_t)b * a.H + h) * a.nchunk + chunk) * D + tid] = t;
+  }
+}
+
+// K mean: sum partials in chunk order (float64), /L, -> fp32 -> input dtype.
+template <int DT>
+__global__ void kmean_finalize_kernel(const double* partial, u16* km, int H, int L, int D, int nchunk,
+                                      const int32_t* cu_seqlens) {
+  const int h = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
+  if (cu_seqlens) L = cu_seqlens[b + 1] - cu_seqlens[b];
+  if (d >= D) return;
+  int nc = (L + kChunkRows - 1) / kChunkRows;
+  double s = 0;
+  for (int c = 0; c < nc; c++) s += partial[(((int64_t)b * H + h) * nchunk + c) * D + d];
+  float m = L > 0 ? (float)(s / (double)L) : 0.f;
+  km[((int64_t)b * H + h) * D + d] = from_f32<DT>(m);
+}
+
+// V scale: max of partial abs-maxima, scale = max(amax/448, 1e-12).
+__global__ void vscale_finalize_kernel(const float* partial, float* vscale, int H, int L, int D, int nchunk,
+                                       const int32_t* cu_seqlens) {
+  const int h = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
+  if (cu_seqlens) L = cu_seqlens[b + 1] - cu_seqlens[b];
+  if (d >= D) return;
+  int nc = (L + kChunkRows - 1) / kChunkRows;
+  float m = 0.f;
+  for (int c = 0; c < nc; c++) m = fmaxf(m, partial[(((int64_t)b * H + h) * nchunk + c) * D + d]);
+  vscale[((int64_t)b * H + h) * D + d] = fmaxf(m / 448.0f, kScaleFloor);
+}
+
+// ---------------------------------------------------------------------------------------------
+// V preparation: one workgroup per panel (128 rows x D of one (batch, head)).
+// Elements are converted, scattered into LDS in panel byte order and streamed out linearly.
+// ---------------------------------------------------------------------------------------------
+
+template <int DT, int D, int PV>
+__global__ void __launch_bounds__(256) prep_v_kernel(PrepVArgs a) {
+  constexpr int TPR = D / 8, RPP = 256 / TPR, NP = kPanelRows / RPP;
+  constexpr int ESZ = (PV == 1) ? 1 : 2;
+  constexpr int PANEL_BYTES = kPanelRows * D * ESZ;
+  __shared__ __attribute__((aligned(16))) uint8_t stage[PANEL_BYTES];
+  const int pidx = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const int tid = threadIdx.x, tr = tid / TPR, tc = tid % TPR;
+  int L = a.L;
+  int64_t vbase, pbase;
+  if (a.cu_seqlens) {
+    int s0 = a.cu_seqlens[b];
+    L = a.cu_seqlens[b + 1] - s0;
+    vbase = (int64_t)s0 * a.v_sn + (int64_t)h * a.v_sh;
+    pbase = ((int64_t)h * a.panel_sh + a.cu_panels[b] + pidx) * PANEL_BYTES;
+  } else {
+    vbase = (int64_t)b * a.v_sb + (int64_t)h * a.v_sh;
+    pbase = (((int64_t)b * a.H + h) * ((L + kPanelRows - 1) / kPanelRows) + pidx) * PANEL_BYTES;
+  }
+  const int n0 = pidx * kPanelRows;
+  if (n0 >= L) return;
+  float sc[8];
+  if constexpr (PV == 1) {
+#pragma unroll
+    for (int i = 0; i < 8; i++) sc[i] = a.vscale[((int64_t)b * a.H + h) * D + tc * 8 + i];
+  }
+#pragma unroll
+  for (int p = 0; p < NP; p++) {
+    int r = p * RPP + tr;
+    uint4 raw = make_uint4(0, 0, 0, 0);
+    if (n0 + r < L) raw = *reinterpret_cast<const uint4*>(a.v + vbase + (int64_t)(n0 + r) * a.v_sn + tc * 8);
+    const u16* e = reinterpret_cast<const u16*>(&raw);
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      float x = to_f32<DT>(e[i]);
+      int d = tc * 8 + i;
+      if constexpr (PV == 1) {
+        float z = x / sc[i];
+        z = fminf(fmaxf(z, -448.f), 448.f);
+        int pk = __builtin_amdgcn_cvt_pk_fp8_f32(z, z, 0, false);
+        stage[panel_index_fp8(r, d, D)] = (uint8_t)(pk & 0xff);
+      } else {
+        reinterpret_cast<u16*>(stage)[panel_index_fp16(r, d, D)] = f32_to_f16(x);
+      }
+    }
+  }
+  __syncthreads();
+  const uint4* src = reinterpret_cast<const uint4*>(stage);
+  uint4* dst = reinterpret_cast<uint4*>(a.panels + pbase);
+#pragma unroll
+  for (int i = 0; i < PANEL_BYTES / 16 / 256; i++) dst[i * 256 + tid] = src[i * 256 + tid];
+}
+
+// ---------------------------------------------------------------------------------------------
+// Host-side launchers (called from the C ABI in sage_api.hip).
+// ---------------------------------------------------------------------------------------------
+hipError_t launch_quant_int8(const QuantArgs& a, int dtype, int max_blocks, hipStream_t st) {
+  dim3 grid(max_blocks, a.H, a.B), block(256);
+  if (dtype == 0 && a.D == 64) quant_int8_kernel<0, 64><<<grid, block, 0, st>>>(a);
+  else if (dtype == 0 && a.D == 128) quant_int8_kernel<0, 128><<<grid, block, 0, st>>>(a);
+  else if (dtype == 1 && a.D == 64) quant_int8_kernel<1, 64><<<grid, block, 0, st>>>(a);
+  else quant_int8_kernel<1, 128><<<grid, block, 0, st>>>(a);
+  return hipGetLastError();
+}
+
+int colstat_chunks(int L) { return (L + kChunkRows - 1) / kChunkRows; }
+
+template <int MODE>
+static hipError_t launch_colstat(const ColStatArgs& a, int dtype, hipStream_t st) {
+  dim3 grid(a.nchunk, a.H, a.B), block(256);
+  if (dtype == 0 && a.D == 64) colstat_partial_kernel<0, 64, MODE><<<grid, block, 0, st>>>(a);
+  else if (dtype == 0 && a.D == 128) colstat_partial_kernel<0, 128, MODE><<<grid, block, 0, st>>>(a);
+  else if (dtype == 1 && a.D == 64) colstat_partial_kernel<1, 64, MODE><<<grid, block, 0, st>>>(a);
+  else colstat_partial_kernel<1, 128, MODE><<<grid, block, 0, st>>>(a);
+  return hipGetLastError();
+}
+
+hipError_t launch_k_mean(const ColStatArgs& a, int dtype, void* km, hipStream_t st) {
+  if (a.nchunk == 0 || a.B == 0 || a.H == 0) return hipSuccess;
+  hipError_t e = launch_colstat<0>(a, dtype, st);
+  if (e != hipSuccess) return e;
+  dim3 grid(a.H, a.B), block(a.D);
+  if (dtype == 0) kmean_finalize_kernel<0><<<grid, block, 0, st>>>((const double*)a.partial, (u16*)km, a.H, a.L, a.D, a.nchunk, a.cu_seqlens);
+  else kmean_finalize_kernel<1><<<grid, block, 0, st>>>((const double*)a.partial, (u16*)km, a.H, a.L, a.D, a.nchunk, a.cu_seqlens);
+  return hipGetLastError();
+}
+
+hipError_t launch_v_scale(const ColStatArgs& a, int dtype, float* vscale, hipStream_t st) {
+  if (a.nchunk == 0 || a.B == 0 || a.H == 0) return hipSuccess;
+  hipError_t e = launch_colstat<1>(a, dtype, st);
+  if (e != hipSuccess) return e;
+  dim3 grid(a.H, a.B), block(a.D);
+  vscale_finalize_kernel<<<grid, block, 0, st>>>((const float*)a.partial, vscale, a.H, a.L, a.D, a.nchunk, a.cu_seqlens);
+  return hipGetLastError();
+}
+
+hipError_t launch_prep_v(const PrepVArgs& a, int dtype, int pv, int max_panels, hipStream_t st) {
+  if (max_panels == 0 || a.B == 0 || a.H == 0) return hipSuccess;
+  dim3 grid(max_panels, a.H, a.B), block(256);
+#define SAGE_PREPV(DT, DD, PVV) prep_v_kernel<DT, DD, PVV><<<grid, block, 0, st>>>(a)
+  if (dtype == 0) {
+    if (a.D == 64) { if (pv) SAGE_PREPV(0, 64, 1); else SAGE_PREPV(0, 64, 0); }
+    else { if (pv) SAGE_PREPV(0, 128, 1); else SAGE_PREPV(0, 128, 0); }
+  } else {
+    if (a.D == 64) { if (pv) SAGE_PREPV(1, 64, 1); else SAGE_PREPV(1, 64, 0); }
+    else { if (pv) SAGE_PREPV(1, 128, 1); else SAGE_PREPV(1, 128, 0); }
+  }
+#undef SAGE_PREPV
+  return hipGetLastError();
+}
+
+}  // namespace sage

@@ -1,0 +1,379 @@
+"""Python entry points of the MI355X SageAttention forward path.
+
+A thin shim over the C ABI (include/sage_mi355x.h): it checks the arguments the way the reference
+wrappers do, allocates outputs and scratch with torch, and passes raw pointers, strides and the
+current HIP stream.  All arithmetic happens in hand-written gfx950 kernels.
+
+Mirrored reference interfaces (same names, argument meaning and error classes):
+  per_block_int8  backends/_enflame/ops/sage_attention/quant_per_block.py:49-101
+                  backends/_hygon/ops/sageattention/sageattention_hip.py:37-51
+  forward         backends/_hygon/ops/sageattention/sageattention_hip.py:54-74
+                  backends/_enflame/ops/sage_attention/attn_qk_int8_per_block_native.py:438-523
+  sageattn        call sites backends/_metax/benchmarks/sage_attention/benchmark.py:29 and
+                  backends/_mthreads/benchmarks/sage_attention_benchmark_compare.py:300-313
+  backend_name    backends/_hygon/ops/sageattention/sageattention_hip.py:77-79
+"""
+from __future__ import annotations
+
+import ctypes
+
+import torch
+
+from . import _cabi
+from ._cabi import DT_BF16, DT_F16, PANEL_ROWS, PV_FP8, PV_FP16, check, lib
+
+__all__ = ["per_block_int8", "forward", "sageattn", "sageattn_varlen", "backend_name", "k_mean", "prepare_v",
+           "per_block_int8_varlen", "varlen_plan"]
+
+_LOG2E_REF = 1.44269504  # quant_per_block.py:87
+
+
+def backend_name() -> str:
+    return lib().sage_backend_name().decode()
+
+
+# ------------------------------------------------------------------------------------------------
+# helpers
+# ------------------------------------------------------------------------------------------------
+def _ptr(t):
+    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+def _stream(t: torch.Tensor):
+    return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def _dt(dtype: torch.dtype) -> int:
+    if dtype == torch.float16:
+        return DT_F16
+    if dtype == torch.bfloat16:
+        return DT_BF16
+    raise TypeError(f"dtype {dtype} is not float16 or bfloat16")
+
+
+def _check_float(name: str, x) -> None:
+    """sageattention_hip.py:30-34."""
+    if not isinstance(x, torch.Tensor) or not x.is_cuda or x.dtype not in (torch.float16, torch.bfloat16):
+        raise TypeError(f"{name} must be a GPU FP16/BF16 tensor")
+    if x.ndim != 4 or not x.is_contiguous():
+        raise ValueError(f"{name} must be contiguous rank 4")
+
+
+def _layout(t: torch.Tensor, tensor_layout: str):
+    """(B, H, L, D, stride_b, stride_h, stride_n), sageattention_triton.py:132-137."""
+    if tensor_layout == "HND":
+        return t.shape[0], t.shape[1], t.shape[2], t.shape[3], t.stride(0), t.stride(1), t.stride(2)
+    if tensor_layout == "NHD":
+        return t.shape[0], t.shape[2], t.shape[1], t.shape[3], t.stride(0), t.stride(2), t.stride(1)
+    raise ValueError(f"tensor_layout {tensor_layout!r} is not supported")
+
+
+def _check_blocks_quant(BLKQ, BLKK):
+    for b in (BLKQ, BLKK):
+        if b not in (16, 32, 64, 128):
+            raise NotImplementedError(f"quantisation block {b} is not supported (16, 32, 64 or 128)")
+
+
+def _q_mult(head_dim: int, sm_scale) -> float:
+    if sm_scale is None:
+        sm_scale = head_dim ** -0.5
+    return float(sm_scale) * _LOG2E_REF
+
+
+# ------------------------------------------------------------------------------------------------
+# quantisers
+# ------------------------------------------------------------------------------------------------
+@torch.no_grad()
+def k_mean(k: torch.Tensor, tensor_layout: str = "HND") -> torch.Tensor:
+    """Per-(batch, kv-head, channel) mean of K over the sequence in k's dtype, shaped to broadcast
+    against k ([B,H,1,D] for HND, [B,1,H,D] for NHD): the `km` argument of per_block_int8."""
+    _check_float("k", k)
+    B, H, L, D, sb, sh, sn = _layout(k, tensor_layout)
+    if D not in (64, 128):
+        raise NotImplementedError("head_dim must be 64 or 128")
+    km = torch.empty((B, H, D), device=k.device, dtype=k.dtype)
+    ws_bytes = lib().sage_k_mean_workspace_bytes(B, H, L, D)
+    ws = torch.empty(max(ws_bytes, 8), device=k.device, dtype=torch.uint8)
+    check(lib().sage_k_mean(_ptr(k), _ptr(km), _ptr(ws), ws_bytes, B, H, L, D, sb, sh, sn, _dt(k.dtype), None, _stream(k)))
+    return km.view(B, H, 1, D) if tensor_layout == "HND" else km.view(B, 1, H, D)
+
+
+def _quant_one(x, km, blk, mult, tensor_layout):
+    B, H, L, D, sb, sh, sn = _layout(x, tensor_layout)
+    out = torch.empty(x.shape, device=x.device, dtype=torch.int8)
+    _, _, _, _, osb, osh, osn = _layout(out, tensor_layout)
+    scale = torch.empty((B, H, (L + blk - 1) // blk), device=x.device, dtype=torch.float32)
+    km_sb = km_sh = 0
+    if km is not None:
+        if km.dtype != x.dtype or km.device != x.device:
+            raise ValueError("km must have k's dtype and device")
+        km = km.expand((B, H, 1, D) if tensor_layout == "HND" else (B, 1, H, D))
+        if km.stride(-1) != 1 and D > 1:
+            km = km.contiguous()
+        km_sb, km_sh = (km.stride(0), km.stride(1)) if tensor_layout == "HND" else (km.stride(0), km.stride(2))
+    check(lib().sage_quant_int8(_ptr(x), _ptr(out), _ptr(scale), _ptr(km), B, H, L, D, sb, sh, sn, osb, osh, osn,
+                                km_sb, km_sh, blk, mult, _dt(x.dtype), None, None, 0, _stream(x)))
+    return out, scale
+
+
+@torch.no_grad()
+def per_block_int8(q, k, km=None, BLKQ=128, BLKK=64, sm_scale=None, tensor_layout="HND"):
+    """Per-block INT8 quantisation of Q and K; returns (q_int8, q_scale, k_int8, k_scale).
+
+    Same contract as quant_per_block.py:49-101: optional ``k - km`` in the input dtype, Q scaled by
+    ``sm_scale * 1.44269504`` (default sm_scale = head_dim**-0.5), K by 1, scales [B, H, ceil(L/BLK)].
+    """
+    _check_float("q", q)
+    _check_float("k", k)
+    if q.dtype != k.dtype or q.device != k.device:
+        raise ValueError("q and k must have the same dtype and device")
+    if tensor_layout not in ("HND", "NHD"):
+        raise ValueError(f"Unknown tensor layout: {tensor_layout}")
+    if q.shape[-1] not in (64, 128):
+        raise NotImplementedError("head_dim must be 64 or 128")
+    if q.shape[-1] != k.shape[-1]:
+        raise ValueError("q and k head dimensions differ")
+    _check_blocks_quant(BLKQ, BLKK)
+    q_int8, q_scale = _quant_one(q, None, BLKQ, _q_mult(q.shape[-1], sm_scale), tensor_layout)
+    k_int8, k_scale = _quant_one(k, km, BLKK, 1.0, tensor_layout)
+    return q_int8, q_scale, k_int8, k_scale
+
+
+@torch.no_grad()
+def prepare_v(v: torch.Tensor, tensor_layout: str = "HND", pv_mode: str = "fp16"):
+    """V -> MFMA-ready panels.  Returns (panels uint8 tensor, v_scale [B,H,D] float32 or None)."""
+    _check_float("v", v)
+    pv = _pv(pv_mode)
+    B, H, L, D, sb, sh, sn = _layout(v, tensor_layout)
+    if D not in (64, 128):
+        raise NotImplementedError("head_dim must be 64 or 128")
+    panels = torch.empty(max(lib().sage_v_panel_bytes(B, H, L, D, pv), 16), device=v.device, dtype=torch.uint8)
+    v_scale = ws = None
+    ws_bytes = 0
+    if pv == PV_FP8:
+        v_scale = torch.empty((B, H, D), device=v.device, dtype=torch.float32)
+        ws_bytes = lib().sage_prep_v_workspace_bytes(B, H, L, D, pv)
+        ws = torch.empty(max(ws_bytes, 8), device=v.device, dtype=torch.uint8)
+    check(lib().sage_prep_v(_ptr(v), _ptr(panels), _ptr(v_scale), _ptr(ws), ws_bytes, B, H, L, D, sb, sh, sn,
+                            _dt(v.dtype), pv, None, None, 0, _stream(v)))
+    return panels, v_scale
+
+
+def _pv(pv_mode) -> int:
+    if pv_mode in ("fp16", PV_FP16, torch.float16):
+        return PV_FP16
+    if pv_mode in ("fp8", PV_FP8, getattr(torch, "float8_e4m3fn", "fp8")):
+        return PV_FP8
+    raise ValueError(f"pv_mode {pv_mode!r} is not 'fp16' or 'fp8'")
+
+
+# ------------------------------------------------------------------------------------------------
+# attention on quantised operands
+# ------------------------------------------------------------------------------------------------
+@torch.no_grad()
+def forward(q, k, v, q_scale, k_scale, tensor_layout="HND", attn_mask=None, output_dtype=torch.float16,
+            return_lse=False, maxnreg=None, block_m=None, num_warps=None, num_stages=None, backend=None,
+            BLKQ=128, BLKK=64, is_causal=False, pv_mode="fp16"):
+    """Fused INT8-QK attention on operands produced by per_block_int8; returns (out, lse).
+
+    Signature of sageattention_hip.py:55-56 / attn_qk_int8_per_block_native.py:438-453; the tuning
+    keywords (maxnreg, block_m, num_warps, num_stages, backend) are accepted and ignored as in
+    sageattention_triton.py:169.  Additions: ``BLKQ``/``BLKK`` name the scale blocks when they are
+    not the reference's 128/64, ``is_causal`` and ``pv_mode`` ("fp16" | "fp8").
+    ``lse`` is base 2 (sageattention_triton.py:127-129) and an empty tensor unless requested.
+    """
+    for name, t in (("q", q), ("k", k)):
+        if not isinstance(t, torch.Tensor) or not t.is_cuda or t.dtype != torch.int8 or not t.is_contiguous():
+            raise TypeError(f"{name} must be contiguous GPU INT8")
+    _check_float("v", v)
+    if q_scale.dtype != torch.float32 or k_scale.dtype != torch.float32:
+        raise TypeError("q_scale and k_scale must be FP32")
+    if output_dtype not in (torch.float16, torch.bfloat16):
+        raise NotImplementedError("output_dtype must be FP16 or BF16")
+    if maxnreg is not None and maxnreg <= 0:
+        raise ValueError("maxnreg must be positive")
+    if attn_mask is not None:
+        raise NotImplementedError("attn_mask is not supported by the MI355X kernel (use is_causal)")
+    if q.ndim != 4 or k.ndim != 4:
+        raise ValueError("q, k, and v must be rank-4 tensors")
+    B, Hq, Sq, D, qsb, qsh, qsn = _layout(q, tensor_layout)
+    Bk, Hkv, Skv, Dk, ksb, ksh, ksn = _layout(k, tensor_layout)
+    Bv, Hv, Sv, Dv, _, _, _ = _layout(v, tensor_layout)
+    if Dk != D or Dv != D or Sv != Skv or Hv != Hkv or Bk != B or Bv != B:
+        raise ValueError("incompatible q/k/v shapes")
+    if Hq % Hkv:
+        raise ValueError("query heads must be divisible by KV heads")
+    if D not in (64, 128):
+        raise NotImplementedError("head_dim must be 64 or 128")
+    if BLKQ % 32 or BLKK % 32 or not (0 < BLKQ <= 128) or not (0 < BLKK <= 128):
+        raise NotImplementedError("the attention kernel needs scale blocks of 32, 64, 96 or 128 rows")
+    exp_q = (B, Hq, (Sq + BLKQ - 1) // BLKQ)
+    exp_k = (B, Hkv, (Skv + BLKK - 1) // BLKK)
+    if tuple(q_scale.shape) != exp_q:
+        raise ValueError(f"q_scale has shape {tuple(q_scale.shape)}, expected {exp_q}")
+    if tuple(k_scale.shape) != exp_k:
+        raise ValueError(f"k_scale has shape {tuple(k_scale.shape)}, expected {exp_k}")
+    if q_scale.device != q.device or k_scale.device != q.device or k.device != q.device or v.device != q.device:
+        raise ValueError("all tensors must be on the same device")
+    pv = _pv(pv_mode)
+    panels, v_scale = prepare_v(v, tensor_layout, pv)
+    out = torch.empty(q.shape, device=q.device, dtype=output_dtype)
+    _, _, _, _, osb, osh, osn = _layout(out, tensor_layout)
+    lse = torch.empty((B, Hq, Sq), device=q.device, dtype=torch.float32) if return_lse else torch.empty(0, device=q.device)
+    check(lib().sage_attn_fwd(_ptr(q), _ptr(k), _ptr(panels), _ptr(q_scale.contiguous()), _ptr(k_scale.contiguous()),
+                              _ptr(v_scale), _ptr(out), _ptr(lse if return_lse else None),
+                              B, Hq, Hkv, Sq, Skv, D, qsb, qsh, qsn, ksb, ksh, ksn, osb, osh, osn,
+                              BLKQ, BLKK, int(bool(is_causal)), pv, _dt(output_dtype),
+                              None, None, None, 0, 0, 0, 0, _stream(q)))
+    return out, lse
+
+
+# ------------------------------------------------------------------------------------------------
+# one-call API
+# ------------------------------------------------------------------------------------------------
+@torch.no_grad()
+def sageattn(q, k, v, tensor_layout="HND", is_causal=False, sm_scale=None, smooth_k=True, pv_mode="fp16",
+             BLKQ=128, BLKK=64, return_lse=False, qk_quant_dtype="int8", quant_recipe=None, **kwargs):
+    """Quantise + attend in one call: out = softmax(q k^T * sm_scale [causal]) v.
+
+    Returns ``out`` (q's shape and dtype), or ``(out, lse)`` with ``return_lse=True`` where lse is
+    the natural-log LSE of the *smoothed* logits (q.(k - mean_k)) * sm_scale.
+    """
+    if qk_quant_dtype != "int8":
+        raise NotImplementedError("only INT8 Q/K quantisation is implemented")
+    if kwargs:
+        raise TypeError(f"unexpected arguments: {sorted(kwargs)}")
+    for name, t in (("q", q), ("k", k), ("v", v)):
+        _check_float(name, t)
+    if not (q.dtype == k.dtype == v.dtype) or not (q.device == k.device == v.device):
+        raise ValueError("q, k and v must have the same dtype and device")
+    B, Hq, Sq, D, qsb, qsh, qsn = _layout(q, tensor_layout)
+    Bk, Hkv, Skv, Dk, ksb, ksh, ksn = _layout(k, tensor_layout)
+    Bv, Hv, Sv, Dv, vsb, vsh, vsn = _layout(v, tensor_layout)
+    if Dk != D or Dv != D or Sv != Skv or Hv != Hkv or Bk != B or Bv != B:
+        raise ValueError("incompatible q/k/v shapes")
+    if Hq % Hkv:
+        raise ValueError("query heads must be divisible by KV heads")
+    if D not in (64, 128):
+        raise NotImplementedError("head_dim must be 64 or 128")
+    if BLKQ % 32 or BLKK % 32 or not (0 < BLKQ <= 128) or not (0 < BLKK <= 128):
+        raise NotImplementedError("the attention kernel needs scale blocks of 32, 64, 96 or 128 rows")
+    pv = _pv(pv_mode)
+    out = torch.empty(q.shape, device=q.device, dtype=q.dtype)
+    _, _, _, _, osb, osh, osn = _layout(out, tensor_layout)
+    lse = torch.empty((B, Hq, Sq), device=q.device, dtype=torch.float32) if return_lse else None
+    ws_bytes = lib().sage_sageattn_workspace_bytes(B, Hq, Hkv, Sq, Skv, D, BLKQ, BLKK, pv, 0, 0, 0)
+    ws = torch.empty(max(ws_bytes, 256), device=q.device, dtype=torch.uint8)
+    check(lib().sage_sageattn(_ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _ptr(ws), ws_bytes,
+                              B, Hq, Hkv, Sq, Skv, D, qsb, qsh, qsn, ksb, ksh, ksn, vsb, vsh, vsn, osb, osh, osn,
+                              _dt(q.dtype), BLKQ, BLKK, float(D ** -0.5 if sm_scale is None else sm_scale),
+                              int(bool(is_causal)), int(bool(smooth_k)), pv, None, None, 0, 0, _stream(q)))
+    if return_lse:
+        return out, lse * 0.6931471805599453
+    return out
+
+
+# ------------------------------------------------------------------------------------------------
+# packed variable-length batches
+# ------------------------------------------------------------------------------------------------
+def _check_packed(name, x):
+    if not isinstance(x, torch.Tensor) or not x.is_cuda or x.dtype not in (torch.float16, torch.bfloat16):
+        raise TypeError(f"{name} must be a GPU FP16/BF16 tensor")
+    if x.ndim != 3 or not x.is_contiguous():
+        raise ValueError(f"{name} must be contiguous [total_tokens, heads, head_dim]")
+
+
+def _check_cu(name, cu, device):
+    if not isinstance(cu, torch.Tensor) or cu.dtype != torch.int32 or cu.ndim != 1 or cu.numel() < 2:
+        raise TypeError(f"{name} must be a 1-D int32 tensor of length nseq+1")
+    if cu.device != device:
+        raise ValueError(f"{name} must be on the same device as q")
+
+
+@torch.no_grad()
+def sageattn_varlen(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, is_causal=False, sm_scale=None,
+                    smooth_k=True, pv_mode="fp16", BLKQ=128, BLKK=64):
+    """Packed variable-length attention: q [Tq, Hq, D], k/v [Tk, Hkv, D], cu_seqlens int32 [nseq+1]
+    on the device.  Quantisation blocks and the K mean restart at every sequence; the (sequence,
+    q-tile) work list is built and cost-ordered on the device, so no host synchronisation happens."""
+    for name, t in (("q", q), ("k", k), ("v", v)):
+        _check_packed(name, t)
+    _check_cu("cu_seqlens_q", cu_seqlens_q, q.device)
+    _check_cu("cu_seqlens_k", cu_seqlens_k, q.device)
+    if cu_seqlens_q.numel() != cu_seqlens_k.numel():
+        raise ValueError("cu_seqlens_q and cu_seqlens_k must describe the same number of sequences")
+    if not (q.dtype == k.dtype == v.dtype) or not (q.device == k.device == v.device):
+        raise ValueError("q, k and v must have the same dtype and device")
+    Tq, Hq, D = q.shape
+    Tk, Hkv, Dk = k.shape
+    if Dk != D or tuple(v.shape) != tuple(k.shape):
+        raise ValueError("incompatible q/k/v shapes")
+    if Hq % Hkv:
+        raise ValueError("query heads must be divisible by KV heads")
+    if D not in (64, 128):
+        raise NotImplementedError("head_dim must be 64 or 128")
+    if BLKQ % 32 or BLKK % 32 or not (0 < BLKQ <= 128) or not (0 < BLKK <= 128):
+        raise NotImplementedError("the attention kernel needs scale blocks of 32, 64, 96 or 128 rows")
+    nseq = cu_seqlens_q.numel() - 1
+    pv = _pv(pv_mode)
+    out = torch.empty_like(q)
+    ws_bytes = lib().sage_sageattn_workspace_bytes(nseq, Hq, Hkv, int(max_seqlen_q), int(max_seqlen_k), D, BLKQ, BLKK, pv,
+                                                   Tq, Tk, 1)
+    ws = torch.empty(max(ws_bytes, 256), device=q.device, dtype=torch.uint8)
+    check(lib().sage_sageattn(_ptr(q), _ptr(k), _ptr(v), _ptr(out), None, _ptr(ws), ws_bytes,
+                              nseq, Hq, Hkv, int(max_seqlen_q), int(max_seqlen_k), D,
+                              0, q.stride(1), q.stride(0), 0, k.stride(1), k.stride(0), 0, v.stride(1), v.stride(0),
+                              0, out.stride(1), out.stride(0),
+                              _dt(q.dtype), BLKQ, BLKK, float(D ** -0.5 if sm_scale is None else sm_scale),
+                              int(bool(is_causal)), int(bool(smooth_k)), pv,
+                              _ptr(cu_seqlens_q), _ptr(cu_seqlens_k), Tq, Tk, _stream(q)))
+    return out
+
+
+@torch.no_grad()
+def varlen_plan(cu_seqlens_q, cu_seqlens_k, total_q, BLKQ=128, BLKK=64, is_causal=False):
+    """Runs the device-side scheduler and returns its raw int32 buffer plus the offsets of
+    (cu_qblk, cu_kblk, cu_panel, tile_count, tiles) inside it."""
+    _check_cu("cu_seqlens_q", cu_seqlens_q, cu_seqlens_q.device)
+    nseq = cu_seqlens_q.numel() - 1
+    n = lib().sage_varlen_plan_ints(nseq, int(total_q))
+    plan = torch.zeros(n, device=cu_seqlens_q.device, dtype=torch.int32)
+    offs = (ctypes.c_int64 * 5)()
+    lib().sage_varlen_plan_offsets(nseq, int(total_q), offs)
+    check(lib().sage_varlen_plan(_ptr(cu_seqlens_q), _ptr(cu_seqlens_k), nseq, int(total_q), BLKQ, BLKK,
+                                 int(bool(is_causal)), _ptr(plan), n, _stream(plan)))
+    return plan, [int(x) for x in offs]
+
+
+@torch.no_grad()
+def per_block_int8_varlen(q, k, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, km=None, BLKQ=128, BLKK=64,
+                          sm_scale=None):
+    """Packed per-block INT8 quantiser: blocks restart at each sequence.  Returns
+    (q_int8, q_scale [Hq, nblk_bound], k_int8, k_scale [Hkv, nblk_bound], plan, plan_offsets); sequence i's
+    blocks start at plan[offs[0] + i] (Q) / plan[offs[1] + i] (K).  ``km`` is [nseq, Hkv, D] or None."""
+    _check_packed("q", q)
+    _check_packed("k", k)
+    _check_blocks_quant(BLKQ, BLKK)
+    Tq, Hq, D = q.shape
+    Tk, Hkv, _ = k.shape
+    nseq = cu_seqlens_q.numel() - 1
+    plan, offs = varlen_plan(cu_seqlens_q, cu_seqlens_k, Tq, BLKQ, BLKK)
+    qi = torch.empty(q.shape, device=q.device, dtype=torch.int8)
+    ki = torch.empty(k.shape, device=k.device, dtype=torch.int8)
+    qs_sh, ks_sh = Tq // BLKQ + nseq, Tk // BLKK + nseq
+    qs = torch.zeros((Hq, qs_sh), device=q.device, dtype=torch.float32)
+    ks = torch.zeros((Hkv, ks_sh), device=q.device, dtype=torch.float32)
+    esz = 4
+    cu_qblk = ctypes.c_void_p(plan.data_ptr() + offs[0] * esz)
+    cu_kblk = ctypes.c_void_p(plan.data_ptr() + offs[1] * esz)
+    check(lib().sage_quant_int8(_ptr(q), _ptr(qi), _ptr(qs), None, nseq, Hq, int(max_seqlen_q), D,
+                                0, q.stride(1), q.stride(0), 0, qi.stride(1), qi.stride(0), 0, 0,
+                                BLKQ, _q_mult(D, sm_scale), _dt(q.dtype), _ptr(cu_seqlens_q), cu_qblk, qs_sh, _stream(q)))
+    km_sb = km_sh = 0
+    if km is not None:
+        km = km.contiguous()
+        km_sb, km_sh = km.stride(0), km.stride(1)
+    check(lib().sage_quant_int8(_ptr(k), _ptr(ki), _ptr(ks), _ptr(km), nseq, Hkv, int(max_seqlen_k), D,
+                                0, k.stride(1), k.stride(0), 0, ki.stride(1), ki.stride(0), km_sb, km_sh,
+                                BLKK, 1.0, _dt(k.dtype), _ptr(cu_seqlens_k), cu_kblk, ks_sh, _stream(k)))
+    return qi, qs, ki, ks, plan, offs
