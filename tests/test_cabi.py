@@ -1,0 +1,95 @@
+"""The C-ABI library loads without a GPU and exports every symbol include/sage_mi355x.h declares;
+argument errors are reported with the documented codes before anything is launched."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from baselinebenchmark_amd import _cabi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "sage_mi355x.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(sage_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_and_binding_agree():
+    names = declared_functions()
+    assert names, "no declarations found"
+    assert sorted(_cabi.SIGNATURES) == names
+
+
+def test_library_exports_every_declared_symbol(sage_lib):
+    for name in declared_functions():
+        assert hasattr(sage_lib, name), name
+
+
+def test_backend_name(sage_lib):
+    assert sage_lib.sage_backend_name().decode() == "mi355x_hip_int8_qk_fp8_fp16_pv"
+
+
+def test_size_queries_do_not_need_a_gpu(sage_lib):
+    # C2 shapes: V panels = B*H*S*D bytes in fp8
+    assert sage_lib.sage_v_panel_bytes(2, 32, 16384, 128, _cabi.PV_FP8) == 2 * 32 * 16384 * 128
+    assert sage_lib.sage_v_panel_bytes(1, 24, 32760, 128, _cabi.PV_FP16) == 24 * 256 * 128 * 128 * 2
+    assert sage_lib.sage_k_mean_workspace_bytes(2, 32, 16384, 128) >= 2 * 32 * 32 * 128 * 8
+    assert sage_lib.sage_sageattn_workspace_bytes(2, 32, 32, 16384, 16384, 128, 64, 128, 1, 0, 0, 0) > 3 * 2 * 32 * 16384 * 128
+    n = sage_lib.sage_varlen_plan_ints(16, 266000)
+    offs = (ctypes.c_int64 * 5)()
+    sage_lib.sage_varlen_plan_offsets(16, 266000, offs)
+    assert list(offs)[:4] == [0, 17, 34, 51] and offs[4] == 52 and n > offs[4] + 266000 // 128
+
+
+NULL = ctypes.c_void_p(0)
+FAKE = ctypes.c_void_p(4096)  # never dereferenced: validation fails first
+
+
+@pytest.mark.parametrize("kwargs,code", [
+    (dict(D=96), _cabi.SAGE_ENOTIMPL),
+    (dict(dtype=7), _cabi.SAGE_ETYPE),
+    (dict(blk=48), _cabi.SAGE_ENOTIMPL),
+    (dict(B=-1), _cabi.SAGE_EINVAL),
+    (dict(x_sn=100), _cabi.SAGE_EINVAL),
+    (dict(x=NULL), _cabi.SAGE_EINVAL),
+])
+def test_quant_argument_errors(sage_lib, kwargs, code):
+    a = dict(x=FAKE, out=FAKE, scale=FAKE, km=NULL, B=1, H=1, L=128, D=128, x_sb=128 * 128, x_sh=128 * 128, x_sn=128,
+             o_sb=128 * 128, o_sh=128 * 128, o_sn=128, km_sb=0, km_sh=0, blk=128, mult=1.0, dtype=0)
+    a.update(kwargs)
+    rc = sage_lib.sage_quant_int8(a["x"], a["out"], a["scale"], a["km"], a["B"], a["H"], a["L"], a["D"], a["x_sb"], a["x_sh"],
+                                  a["x_sn"], a["o_sb"], a["o_sh"], a["o_sn"], a["km_sb"], a["km_sh"], a["blk"], a["mult"],
+                                  a["dtype"], NULL, NULL, 0, NULL)
+    assert rc == code
+    assert sage_lib.sage_last_error().decode() != ""
+    with pytest.raises({_cabi.SAGE_EINVAL: ValueError, _cabi.SAGE_ETYPE: TypeError, _cabi.SAGE_ENOTIMPL: NotImplementedError}[code]):
+        _cabi.check(rc)
+
+
+def test_attn_argument_errors(sage_lib):
+    def call(Hq=4, Hkv=2, D=128, blkq=128, blkk=64, pv=0, vs=NULL):
+        return sage_lib.sage_attn_fwd(FAKE, FAKE, FAKE, FAKE, FAKE, vs, FAKE, NULL, 1, Hq, Hkv, 128, 128, D,
+                                      0, 128 * D, D, 0, 128 * D, D, 0, 128 * D, D, blkq, blkk, 0, pv, 0,
+                                      NULL, NULL, NULL, 0, 0, 0, 0, NULL)
+    assert call(Hq=3) == _cabi.SAGE_EINVAL          # heads not divisible
+    assert call(D=32) == _cabi.SAGE_ENOTIMPL
+    assert call(blkk=16) == _cabi.SAGE_ENOTIMPL      # attention needs scale blocks that are multiples of 32
+    assert call(pv=1) == _cabi.SAGE_EINVAL           # fp8 needs v_scale
+    assert call(pv=5) == _cabi.SAGE_EINVAL
+
+
+def test_empty_problem_is_a_no_op(sage_lib):
+    rc = sage_lib.sage_quant_int8(NULL, NULL, NULL, NULL, 0, 4, 128, 128, 0, 0, 128, 0, 0, 128, 0, 0, 128, 1.0, 0,
+                                  NULL, NULL, 0, NULL)
+    assert rc == _cabi.SAGE_OK
+
+
+def test_missing_library_is_loud(monkeypatch, tmp_path):
+    monkeypatch.setattr(_cabi, "_lib", None)
+    monkeypatch.setattr(_cabi, "LIB_PATH", tmp_path / "nope.so")
+    with pytest.raises(_cabi.SageLibraryMissing):
+        _cabi.lib()

@@ -1,0 +1,187 @@
+"""GPU parity of the HIP quantisers against the CPU oracle, through the C ABI.  Bit-exact bar."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import baselinebenchmark_amd as sa
+from oracle import quant as oq
+from tests.helpers import golden_case, randn
+
+pytestmark = [pytest.mark.gpu, pytest.mark.sage_attention]
+DEV = "cuda"
+
+
+def _cmp(q, k, km=None, layout="HND", BLKQ=128, BLKK=64, sm_scale=None):
+    out = sa.per_block_int8(q.to(DEV), k.to(DEV), km=None if km is None else km.to(DEV), BLKQ=BLKQ, BLKK=BLKK,
+                            sm_scale=sm_scale, tensor_layout=layout)
+    ref = oq.per_block_int8(q, k, km=km, BLKQ=BLKQ, BLKK=BLKK, sm_scale=sm_scale, tensor_layout=layout)
+    torch.cuda.synchronize()
+    for name, a, b in zip(("q_int8", "q_scale", "k_int8", "k_scale"), out, ref):
+        assert a.dtype == b.dtype and tuple(a.shape) == tuple(b.shape), name
+        assert torch.equal(a.cpu(), b), f"{name}: {(a.cpu() != b).sum().item()} mismatches"
+    return out
+
+
+def test_reference_golden_vectors(golden):
+    for name in golden["cases"]:
+        c = golden_case(golden, str(name))
+        out = sa.per_block_int8(c["q"].to(DEV), c["k"].to(DEV), km=None if c["km"] is None else c["km"].to(DEV),
+                                BLKQ=c["BLKQ"], BLKK=c["BLKK"], sm_scale=c["sm_scale"], tensor_layout=c["layout"])
+        for key, t in zip(("qi", "qs", "ki", "ks"), out):
+            assert torch.equal(t.cpu(), c[key]), (name, key)
+
+
+@pytest.mark.parametrize("layout", ["HND", "NHD"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("blocks", [(128, 64), (64, 128), (128, 128), (32, 16)])
+def test_bit_exact_random(layout, dtype, D, blocks):
+    g = torch.Generator().manual_seed(2026 + D + blocks[0])
+    q = randn(layout, 2, 3, 333, D, dtype, g)
+    k = randn(layout, 2, 3, 270, D, dtype, g, offset_std=2.0)
+    _cmp(q, k, layout=layout, BLKQ=blocks[0], BLKK=blocks[1])
+
+
+@pytest.mark.parametrize("layout", ["HND", "NHD"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_reference_test_shapes_tail_and_gqa(layout, dtype):
+    # 129 x 70 with 2 q-heads over 1 kv-head: backends/_enflame/test/test_sage_attention_native.py:133-134
+    g = torch.Generator().manual_seed(9)
+    q = randn(layout, 1, 2, 129, 128, dtype, g)
+    k = randn(layout, 1, 1, 70, 128, dtype, g)
+    _cmp(q, k, layout=layout)
+    _cmp(q, k, layout=layout, sm_scale=0.3)
+
+
+@pytest.mark.parametrize("layout", ["HND", "NHD"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_k_mean_and_smoothed_quantisation(layout, dtype):
+    g = torch.Generator().manual_seed(21)
+    q = randn(layout, 2, 4, 700, 128, dtype, g)
+    k = randn(layout, 2, 2, 1300, 128, dtype, g, offset_std=2.0)
+    km = sa.k_mean(k.to(DEV), layout)
+    km_ref = oq.k_mean(k, layout)
+    assert km.dtype == dtype and tuple(km.shape) == tuple(km_ref.shape)
+    assert torch.equal(km.cpu(), km_ref)
+    _cmp(q, k, km=km_ref, layout=layout)
+
+
+def test_adversarial_values():
+    # ties at .5, +-max, zeros, a zero tile, tiny values below the scale floor and huge magnitudes
+    g = torch.Generator().manual_seed(33)
+    D = 64
+    x = (torch.randint(-253, 254, (1, 1, 128 * 6, D), generator=g).float() * 0.5)
+    x[0, 0, 0, 0] = 127.0                       # tile 0: scale exactly 1 -> quotient ties
+    x[0, 0, 128:256] = 0.0                      # tile 1: all zeros -> floor scale
+    x[0, 0, 256:384] *= 1e-30                   # tile 2: tiny values
+    x[0, 0, 384:512] *= 1e30                    # tile 3: huge values
+    x[0, 0, 512:640] = torch.randn((128, D), generator=g) * 10
+    x[0, 0, 512, 0] = 300.0
+    xb = x.to(torch.bfloat16)
+    _cmp(xb, xb.clone(), BLKQ=128, BLKK=128, sm_scale=1.0 / 1.44269504)
+    xh = x.clamp(-6e4, 6e4).to(torch.float16)
+    _cmp(xh, xh.clone(), BLKQ=64, BLKK=32, sm_scale=1.0 / 1.44269504)
+
+
+def test_scale_with_all_ones_significand_takes_the_exact_path():
+    # amax = 127 * 1.9999999 (bf16 cannot hold it, fp16 neither) -> build it through the multiplier:
+    # x = 127 (exact), mult = 1.9999999 -> x32 = 253.99998, scale = RN(253.99998/127) = 1.9999999
+    allones = float(np.frombuffer(np.uint32(0x3FFFFFFF).tobytes(), dtype=np.float32)[0])
+    g = torch.Generator().manual_seed(1)
+    x = torch.randint(-127, 128, (1, 2, 256, 128), generator=g).float()
+    x[..., 0, 0] = 127.0
+    x[..., 128, 0] = -127.0
+    xh = x.half()
+    out = _cmp(xh, xh, BLKQ=128, BLKK=64, sm_scale=allones / 1.44269504)
+    bits = out[1].cpu().numpy().view(np.uint32)
+    assert (bits & 0x7FFFFF == 0x7FFFFF).any(), "the test did not produce an all-ones significand"
+
+
+def test_inputs_are_not_mutated():
+    # backends/_metax/test/sage_attention/test_official_wheel.py:20-32
+    g = torch.Generator().manual_seed(4)
+    q = randn("HND", 1, 2, 256, 128, torch.float16, g).to(DEV)
+    k = randn("HND", 1, 2, 256, 128, torch.float16, g).to(DEV)
+    q0, k0 = q.clone(), k.clone()
+    km = sa.k_mean(k)
+    sa.per_block_int8(q, k, km=km)
+    torch.cuda.synchronize()
+    assert torch.equal(q, q0) and torch.equal(k, k0)
+
+
+def test_full_size_north_star_operand_properties():
+    # BASELINE config 2 operand: [2, 32, 16384, 128] bf16 with per-channel K offsets, Q blk 64 / K blk 128.
+    # Size-independent properties on the whole tensor + oracle equality on two (batch, head) slices.
+    g = torch.Generator(device=DEV).manual_seed(2)
+    B, H, S, D = 2, 32, 16384, 128
+    q = torch.randn((B, H, S, D), device=DEV, generator=g, dtype=torch.float32).to(torch.bfloat16)
+    k = (torch.randn((B, H, S, D), device=DEV, generator=g, dtype=torch.float32)
+         + 2.0 * torch.randn((1, H, 1, D), device=DEV, generator=g, dtype=torch.float32)).to(torch.bfloat16)
+    km = sa.k_mean(k)
+    qi, qs, ki, ks = sa.per_block_int8(q, k, km=km, BLKQ=64, BLKK=128)
+    assert qs.shape == (B, H, S // 64) and ks.shape == (B, H, S // 128)
+    assert int(qi.abs().amax()) == 127 and int(ki.abs().amax()) == 127
+    # every tile's largest magnitude is exactly 127
+    assert torch.all(qi.view(B, H, S // 64, 64 * D).abs().amax(dim=-1) == 127)
+    assert torch.all(ki.view(B, H, S // 128, 128 * D).abs().amax(dim=-1) == 127)
+    # half-step reconstruction bound on K (smoothed input)
+    ksm = (k - km).float()
+    err = (ksm - ki.float() * ks.repeat_interleave(128, dim=-1)[..., None]).abs()
+    assert torch.all(err <= ks.repeat_interleave(128, dim=-1)[..., None] * (0.5 + 1e-5))
+    for (b, h) in ((0, 0), (1, 31)):
+        qq, kk = q[b:b + 1, h:h + 1].cpu(), k[b:b + 1, h:h + 1].cpu()
+        kmr = oq.k_mean(kk)
+        assert torch.equal(kmr, km[b:b + 1, h:h + 1].cpu())
+        r = oq.per_block_int8(qq, kk, km=kmr, BLKQ=64, BLKK=128)
+        assert torch.equal(r[0], qi[b:b + 1, h:h + 1].cpu()) and torch.equal(r[1], qs[b:b + 1, h:h + 1].cpu())
+        assert torch.equal(r[2], ki[b:b + 1, h:h + 1].cpu()) and torch.equal(r[3], ks[b:b + 1, h:h + 1].cpu())
+
+
+@pytest.mark.parametrize("layout", ["HND", "NHD"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("D", [64, 128])
+def test_v_fp8_quantiser_bit_exact(layout, dtype, D):
+    from baselinebenchmark_amd.csrc_layout import unpack_panels
+    g = torch.Generator().manual_seed(17 + D)
+    v = randn(layout, 2, 2, 300, D, dtype, g)
+    v[..., 5] *= 20  # an outlier channel
+    panels, vs = sa.prepare_v(v.to(DEV), layout, "fp8")
+    ref8, refs = oq.quant_v_fp8(v, layout)
+    assert torch.equal(vs.cpu(), refs)
+    got = unpack_panels(panels.cpu(), 2, 2, 300, D, "fp8")              # [B,H,L,D] uint8
+    want = ref8.view(torch.uint8)
+    want = want if layout == "HND" else want.transpose(1, 2)
+    assert torch.equal(got[:, :, :300], want)
+    assert torch.all(got[:, :, 300:] == 0)                              # padded rows are zero
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_v_fp16_panels(dtype):
+    from baselinebenchmark_amd.csrc_layout import unpack_panels
+    g = torch.Generator().manual_seed(18)
+    v = randn("NHD", 1, 2, 129, 64, dtype, g)
+    panels, vs = sa.prepare_v(v.to(DEV), "NHD", "fp16")
+    assert vs is None
+    got = unpack_panels(panels.cpu(), 1, 2, 129, 64, "fp16")            # [B,H,Lpad,D] fp16
+    assert torch.equal(got[:, :, :129], v.transpose(1, 2).to(torch.float16))
+    assert torch.all(got[:, :, 129:] == 0)
+
+
+def test_varlen_quantiser_matches_per_sequence_oracle():
+    g = torch.Generator().manual_seed(41)
+    lens = [70, 129, 513, 1, 256]
+    cu = torch.tensor(np.concatenate([[0], np.cumsum(lens)]), dtype=torch.int32)
+    T = int(cu[-1])
+    q = torch.randn((T, 4, 128), generator=g).to(torch.bfloat16)
+    k = (torch.randn((T, 2, 128), generator=g) + 2.0).to(torch.bfloat16)
+    qi, qs, ki, ks, plan, offs = sa.per_block_int8_varlen(q.to(DEV), k.to(DEV), cu.to(DEV), cu.to(DEV), max(lens), max(lens),
+                                                          BLKQ=64, BLKK=128)
+    r = oq.per_block_int8_varlen(q, k, cu.numpy(), cu.numpy(), BLKQ=64, BLKK=128)
+    nq, nk = r[1].shape[1], r[3].shape[1]
+    assert torch.equal(qi.cpu(), r[0]) and torch.equal(ki.cpu(), r[2])
+    assert torch.equal(qs.cpu()[:, :nq], r[1]) and torch.equal(ks.cpu()[:, :nk], r[3])
+    p = plan.cpu().numpy()
+    assert p[offs[0]:offs[0] + 6].tolist() == oq.seq_block_offsets(cu.numpy(), 64).tolist()
+    assert p[offs[1]:offs[1] + 6].tolist() == oq.seq_block_offsets(cu.numpy(), 128).tolist()

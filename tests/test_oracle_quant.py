@@ -1,0 +1,198 @@
+"""Pins the CPU oracle of the INT8 quantiser (oracle/quant.py) without a GPU.
+
+Evidence, in order of independence:
+ 1. golden vectors produced by the reference's own per_block_int8 under Triton's CPU interpreter
+    (tests/golden/make_quant_golden.py) -- bit-exact;
+ 2. an exact-rational restatement (fractions.Fraction, correctly rounded by construction) of
+    quant_per_block.py:38-46 on small tiles -- catches a reciprocal-multiply or a wrong tie rule;
+ 3. closed-form invariants (arg-max -> +-127, half-step error bound, tail rows ignored).
+"""
+import math
+from fractions import Fraction
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import quant as oq
+from tests.helpers import golden_case, randn
+
+
+# ---------------------------------------------------------------- 1. golden vectors
+def test_oracle_matches_reference_golden(golden):
+    for name in golden["cases"]:
+        c = golden_case(golden, str(name))
+        qi, qs, ki, ks = oq.per_block_int8(c["q"], c["k"], km=c["km"], BLKQ=c["BLKQ"], BLKK=c["BLKK"],
+                                           sm_scale=c["sm_scale"], tensor_layout=c["layout"])
+        assert torch.equal(qi, c["qi"]), name
+        assert torch.equal(ki, c["ki"]), name
+        assert torch.equal(qs, c["qs"]), name
+        assert torch.equal(ks, c["ks"]), name
+
+
+# ---------------------------------------------------------------- 2. exact rational restatement
+def _rn32(fr: Fraction) -> np.float32:
+    """Round an exact rational to the nearest binary32 (ties to even), no intermediate rounding."""
+    if fr == 0:
+        return np.float32(0.0)
+    sign = -1 if fr < 0 else 1
+    a = abs(fr)
+    e = math.floor(math.log2(a)) if a >= 1 else -math.ceil(-math.log2(float(a)) - 1e-12)
+    while Fraction(2) ** e > a:
+        e -= 1
+    while Fraction(2) ** (e + 1) <= a:
+        e += 1
+    e = max(e, -126)
+    ulp = Fraction(2) ** (e - 23)
+    n = a / ulp
+    fl = n.numerator // n.denominator
+    rem = n - fl
+    if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and fl % 2 == 1):
+        fl += 1
+    return np.float32(sign * float(fl * ulp))
+
+
+def _tile_rational(x32, mult):
+    xs = [_rn32(Fraction(float(v)) * Fraction(float(np.float32(mult)))) for v in x32.ravel()]
+    amax = max(abs(float(v)) for v in xs)
+    scale = _rn32(Fraction(amax) / 127)
+    scale = max(scale, np.float32(1e-12))
+    out = []
+    for v in xs:
+        z = _rn32(Fraction(float(v)) / Fraction(float(scale)))
+        z = _rn32(Fraction(float(z)) + (Fraction(1, 2) if z >= 0 else Fraction(-1, 2)))
+        out.append(int(math.trunc(float(z))))
+    return np.array(out, dtype=np.int64).reshape(x32.shape), scale
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("mult", [1.0, 128 ** -0.5 * 1.44269504, 0.3])
+def test_oracle_tile_equals_exact_rational(dtype, mult):
+    g = torch.Generator().manual_seed(7)
+    x = (torch.randn((24, 16), generator=g) * 3).to(dtype)
+    x32 = x.float().numpy()
+    q, s = oq.quant_tile_int8(x32, mult)
+    qr, sr = _tile_rational(x32, mult)
+    assert s == sr
+    assert np.array_equal(q.astype(np.int64), qr)
+
+
+def test_round_half_away_from_zero_ties():
+    # tile max 127 -> scale exactly 1 -> quotients are the inputs: k + 0.5 must round away from zero
+    x = np.array([[127.0, 0.5, -0.5, 1.5, -1.5, 2.5, -2.5, 126.5, -126.5, 0.0, -0.0, 0.49999997]], np.float32)
+    q, s = oq.quant_tile_int8(x, 1.0)
+    assert s == np.float32(1.0)
+    # the last one is the add-then-truncate artefact the reference has (quant_per_block.py:43-44):
+    # 0.49999997 + 0.5 rounds up to 1.0 in binary32, so it quantises to 1, not 0
+    assert q.tolist() == [[127, 1, -1, 2, -2, 3, -3, 127, -127, 0, 0, 1]]
+
+
+# ---------------------------------------------------------------- 3. invariants
+@pytest.mark.parametrize("layout", ["HND", "NHD"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_invariants(layout, dtype):
+    g = torch.Generator().manual_seed(11)
+    B, H, L, D, blk = 2, 3, 200, 64, 64
+    q = randn(layout, B, H, L, D, dtype, g)
+    k = randn(layout, B, H, L, D, dtype, g, offset_std=2.0)
+    qi, qs, ki, ks = oq.per_block_int8(q, k, BLKQ=blk, BLKK=blk, tensor_layout=layout)
+    assert qs.shape == (B, H, math.ceil(L / blk)) and qs.dtype == torch.float32
+    for x, xi, xs, mult in ((q, qi, qs, oq.q_multiplier(D)), (k, ki, ks, np.float32(1.0))):
+        x32 = (x.float() if layout == "HND" else x.float().transpose(1, 2)).numpy() * np.float32(mult)
+        xi_h = (xi if layout == "HND" else xi.transpose(1, 2)).numpy().astype(np.int32)
+        assert np.abs(xi_h).max() <= 127
+        rows = np.repeat(xs.numpy(), blk, axis=-1)[..., :L, None]
+        # half-step bound (+1 ulp of the quotient)
+        assert np.all(np.abs(x32 - xi_h * rows) <= rows * (0.5 + 1e-5))
+        # the arg-max element of every tile maps to +-127 and scale = amax/127
+        for b in range(B):
+            for h in range(H):
+                for t in range(math.ceil(L / blk)):
+                    tile = x32[b, h, t * blk:(t + 1) * blk]
+                    ti = xi_h[b, h, t * blk:(t + 1) * blk]
+                    i = np.unravel_index(np.argmax(np.abs(tile)), tile.shape)
+                    assert abs(ti[i]) == 127
+                    assert xs[b, h, t].item() == np.float32(np.abs(tile).max()) / np.float32(127)
+
+
+def test_tail_rows_do_not_leak_into_scale():
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn((1, 1, 70, 64), generator=g).half()
+    big = torch.cat([x, torch.full((1, 1, 58, 64), 1000.0).half()], dim=2)  # what a padded load would see
+    qi, qs, _, _ = oq.per_block_int8(x, x, BLKQ=128, BLKK=64)
+    qi2, qs2, _, _ = oq.per_block_int8(big, big, BLKQ=128, BLKK=64)
+    assert not torch.equal(qs, qs2[..., :1])  # sanity: the padding would have changed the scale
+    assert qi.shape == x.shape and qs.shape == (1, 1, 1)
+
+
+def test_zero_tile_gets_floor_scale():
+    x = torch.zeros((1, 1, 64, 64), dtype=torch.float16)
+    qi, qs, ki, ks = oq.per_block_int8(x, x, BLKQ=64, BLKK=64)
+    assert torch.all(qi == 0) and torch.all(ki == 0)
+    assert qs.item() == np.float32(1e-12) and ks.item() == np.float32(1e-12)
+
+
+def test_q_multiplier_matches_full_precision_log2e_for_supported_head_dims():
+    for d in (64, 128):
+        assert oq.q_multiplier(d) == np.float32(d ** -0.5 * 1.4426950408889634)
+
+
+def test_exhaustive_fp16_values_single_tile():
+    # every finite fp16 value once, in tiles of 128x64: vectorised oracle == per-tile oracle
+    bits = np.arange(65536, dtype=np.uint16)
+    vals = torch.from_numpy(bits.view(np.int16)).view(torch.float16)
+    vals = vals[torch.isfinite(vals)]
+    n = (vals.numel() // (128 * 64)) * 128 * 64
+    x = vals[:n].reshape(1, 1, -1, 64)
+    qi, qs, _, _ = oq.per_block_int8(x, x, BLKQ=128, BLKK=128, sm_scale=1.0 / 1.44269504)
+    x32 = x.float().numpy()[0, 0]
+    for t in range(x32.shape[0] // 128):
+        q, s = oq.quant_tile_int8(x32[t * 128:(t + 1) * 128], np.float32(1.0 / 1.44269504 * 1.44269504))
+        assert s == qs[0, 0, t].item()
+        assert np.array_equal(q, qi[0, 0, t * 128:(t + 1) * 128].numpy())
+
+
+def test_k_mean_definition():
+    g = torch.Generator().manual_seed(5)
+    k = randn("NHD", 2, 3, 333, 64, torch.bfloat16, g, offset_std=2.0)
+    km = oq.k_mean(k, "NHD")
+    assert km.shape == (2, 1, 3, 64) and km.dtype == torch.bfloat16
+    ref = k.double().mean(dim=1, keepdim=True)
+    assert torch.all((km.double() - ref).abs() <= ref.abs() * 2 ** -8 + 1e-30)
+
+
+def test_fp8_value_set_matches_reference_bit_decoder():
+    # restates the bit layout of backends/_enflame/ops/hpc_ops_attention/fp8_utils.py:19-38
+    bits = torch.arange(256, dtype=torch.int16).to(torch.uint8)
+    vals = bits.view(torch.float8_e4m3fn).float()
+    for b in range(256):
+        s, e, m = b >> 7, (b >> 3) & 15, b & 7
+        if e == 15 and m == 7:
+            assert math.isnan(vals[b].item())
+            continue
+        mag = (m / 8.0) * 2.0 ** -6 if e == 0 else (1 + m / 8.0) * 2.0 ** (e - 7)
+        assert vals[b].item() == (-mag if s else mag)
+
+
+def test_quant_v_fp8_roundtrip_error_bound():
+    g = torch.Generator().manual_seed(9)
+    v = randn("HND", 1, 2, 300, 64, torch.bfloat16, g)
+    v8, sc = oq.quant_v_fp8(v, "HND")
+    assert v8.dtype == torch.float8_e4m3fn and sc.shape == (1, 2, 64)
+    deq = v8.float() * sc[:, :, None, :]
+    err = (deq - v.float()).abs()
+    assert torch.all(err <= v.float().abs() * 2 ** -4 + sc[:, :, None, :] * 2 ** -9)
+    assert torch.all(v8.float().abs().amax(dim=2) == 448.0)
+
+
+def test_varlen_equals_per_sequence():
+    g = torch.Generator().manual_seed(13)
+    lens = [70, 129, 256, 1]
+    cu = np.concatenate([[0], np.cumsum(lens)])
+    q = torch.randn((sum(lens), 2, 64), generator=g).half()
+    k = torch.randn((sum(lens), 1, 64), generator=g).half()
+    qi, qs, ki, ks = oq.per_block_int8_varlen(q, k, cu, cu, BLKQ=128, BLKK=64)
+    offq = oq.seq_block_offsets(cu, 128)
+    assert offq.tolist() == [0, 1, 3, 5, 6]
+    a, b, c, d = oq.per_block_int8(q[70:199].unsqueeze(0), k[70:199].unsqueeze(0), tensor_layout="NHD")
+    assert torch.equal(qi[70:199], a[0]) and torch.equal(qs[:, 1:3], b[0])
