@@ -8,6 +8,7 @@
 #include <cstdio>
 #include <cstring>
 #include <cmath>
+#include <cstdlib>
 
 using namespace sage;
 
@@ -30,6 +31,8 @@ int hip_fail(hipError_t e, const char* what) {
 inline size_t align_up(size_t x, size_t a = 256) { return (x + a - 1) / a * a; }
 
 bool valid_blk_quant(int blk) { return blk == 16 || blk == 32 || blk == 64 || blk == 128; }
+bool valid_blk_attn(int blk) { return blk == 32 || blk == 64 || blk == 128; }
+int ilog2(int x) { int r = 0; while ((1 << r) < x) r++; return r; }
 
 int check_common(int B, int H, int L, int D, int dtype) {
   if (B < 0 || H < 0 || L < 0) return fail(SAGE_EINVAL, "negative dimension (B=%d H=%d L=%d)", B, H, L);
@@ -166,8 +169,8 @@ int sage_attn_fwd(const int8_t* q, const int8_t* k, const void* v_panels, const 
   if (Hkv <= 0 || Hq % Hkv) return fail(SAGE_EINVAL, "query heads (%d) must be divisible by KV heads (%d)", Hq, Hkv);
   if (Skv < 0) return fail(SAGE_EINVAL, "negative kv length");
   if (pv_mode != SAGE_PV_FP16 && pv_mode != SAGE_PV_FP8) return fail(SAGE_EINVAL, "pv_mode %d unknown", pv_mode);
-  if (blkq % 32 || blkk % 32 || blkq <= 0 || blkk <= 0 || blkq > 128 || blkk > 128)
-    return fail(SAGE_ENOTIMPL, "attention needs scale blocks that are multiples of 32 up to 128 (got %d/%d)", blkq, blkk);
+  if (!valid_blk_attn(blkq) || !valid_blk_attn(blkk))
+    return fail(SAGE_ENOTIMPL, "attention needs scale blocks of 32, 64 or 128 rows (got %d/%d)", blkq, blkk);
   if (B == 0 || Hq == 0 || Sq == 0) return SAGE_OK;
   if (!q || !k || !v_panels || !q_scale || !k_scale || !out) return fail(SAGE_EINVAL, "null tensor pointer");
   if (pv_mode == SAGE_PV_FP8 && !v_scale) return fail(SAGE_EINVAL, "fp8 P.V needs v_scale");
@@ -187,8 +190,9 @@ int sage_attn_fwd(const int8_t* q, const int8_t* k, const void* v_panels, const 
   a.B = B; a.Hq = Hq; a.Hkv = Hkv; a.Sq = Sq; a.Skv = Skv;
   a.q_sb = q_sb; a.q_sh = q_sh; a.q_sn = q_sn; a.k_sb = k_sb; a.k_sh = k_sh; a.k_sn = k_sn;
   a.o_sb = o_sb; a.o_sh = o_sh; a.o_sn = o_sn;
-  a.blkq = blkq; a.blkk = blkk; a.out_bf16 = out_dtype == SAGE_DT_BF16;
+  a.blkq = blkq; a.blkk = blkk; a.blkq_shift = ilog2(blkq); a.blkk_shift = ilog2(blkk); a.out_bf16 = out_dtype == SAGE_DT_BF16;
   a.nqt = (Sq + BM - 1) / BM;
+  { const char* e = getenv("SAGE_PP_SPLIT"); a.pp_split = e ? atoi(e) : 0; }
   int64_t grid;
   if (packed) {
     SagePlanLayout L = plan_layout(B, total_q);
@@ -255,8 +259,8 @@ int sage_sageattn(const void* q, const void* k, const void* v, void* out, float*
                   const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k, int total_q, int total_k, sage_stream_t stream) {
   if (int rc = check_common(B, Hq, Sq, D, dtype)) return rc;
   if (Hkv <= 0 || Hq % Hkv) return fail(SAGE_EINVAL, "query heads (%d) must be divisible by KV heads (%d)", Hq, Hkv);
-  if (blkq % 32 || blkk % 32 || blkq <= 0 || blkk <= 0 || blkq > 128 || blkk > 128)
-    return fail(SAGE_ENOTIMPL, "scale blocks must be multiples of 32 up to 128 (got %d/%d)", blkq, blkk);
+  if (!valid_blk_attn(blkq) || !valid_blk_attn(blkk))
+    return fail(SAGE_ENOTIMPL, "scale blocks must be 32, 64 or 128 rows (got %d/%d)", blkq, blkk);
   if (pv_mode != SAGE_PV_FP16 && pv_mode != SAGE_PV_FP8) return fail(SAGE_EINVAL, "pv_mode %d unknown", pv_mode);
   const int varlen = cu_seqlens_q != nullptr;
   if (varlen && !cu_seqlens_k) return fail(SAGE_EINVAL, "packed mode needs cu_seqlens_k");

@@ -23,6 +23,7 @@
 //     with a static 2^kPShift so that fp8's range [2^-9, 448] is used.
 //   * K/V tiles go global -> registers -> LDS, double buffered, one barrier per KV tile.
 #include "sage_launch.h"
+#include <cstdlib>
 
 namespace sage {
 
@@ -62,6 +63,12 @@ __device__ inline float xchg32_sum(float x) {
   return lo + hi;
 }
 
+// Workgroup barrier that only orders LDS traffic: waits for this wavefront's outstanding LDS
+// operations, then s_barrier (global-memory traffic issued ahead stays in flight).
+__device__ inline void lds_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 // 16-byte-chunk swizzle of a K row in LDS: consecutive rows read the same logical chunk from
 // different bank groups (64 banks x 4 bytes = 256 bytes per bank row).
 template <int D>
@@ -80,14 +87,14 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
   constexpr int VESZ = PV ? 1 : 2;
   constexpr int KBYTES = BN * D, VBYTES = BN * D * VESZ, STAGE = KBYTES + VBYTES;
   constexpr int KCHUNKS = KBYTES / 16, VCHUNKS = VBYTES / 16;
-  constexpr int KCH = (KCHUNKS + NTHR - 1) / NTHR, VCH = (VCHUNKS + NTHR - 1) / NTHR;
   constexpr int PANEL_BYTES = kPanelRows * D * VESZ;
   constexpr int CPR = D / 16;
   constexpr float TAU = PCfg<PV>::tau, PSHIFT = PCfg<PV>::pshift;
 
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
-  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);  // wavefront index: uniform, keep it scalar
   const int m = lane & 31, h = lane >> 5;
 
   // ---- which tile am I: heaviest q-tiles first; q-heads sharing a KV head on one XCD ----
@@ -147,7 +154,7 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) qreg[ks] = *reinterpret_cast<const v4i*>(qp + 32 * ks);
   }
-  const float qscale = qsp[min(row0, Lq - 1) / a.blkq];
+  const float qscale = qsp[min(row0, Lq - 1) >> a.blkq_shift];
 
   v16i bias;
 #pragma unroll
@@ -161,34 +168,31 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
     for (int i = 0; i < 16; i++) o[dt][i] = 0.f;
   float m_used = kMInit, lsum = 0.f;
 
-  // ---- cooperative tile loads: global -> registers, registers -> LDS ----
-  v4i kst[KCH], vst[VCH];
-  auto load_tile = [&](int j) {
-    const int n0 = j * BN;
-#pragma unroll
-    for (int i = 0; i < KCH; i++) {
-      int c = i * NTHR + tid, n = c / CPR, cc = c % CPR;
-      int row = min(n0 + n, Lk - 1);
-      if (KCHUNKS % NTHR == 0 || c < KCHUNKS)
-        kst[i] = *reinterpret_cast<const v4i*>(a.k + koff + (int64_t)row * a.k_sn + 16 * cc);
-    }
-    const uint8_t* vsrc = vbase + (int64_t)n0 * D * VESZ;
-#pragma unroll
-    for (int i = 0; i < VCH; i++)
-      if (VCHUNKS % NTHR == 0 || i * NTHR + tid < VCHUNKS)
-        vst[i] = *reinterpret_cast<const v4i*>(vsrc + (int64_t)(i * NTHR + tid) * 16);
+  // ---- tile loads: global memory -> LDS directly (no registers), 1 KB per wavefront instruction ----
+  // Lane l of a wavefront writes LDS bytes [16*l, 16*l+16) of the 1 KB piece, so the K swizzle is
+  // applied on the global side: the lane fetches the 16-byte chunk that belongs in its slot.
+  // Stages form a ring of NSTAGE tiles; the load of tile j+NSTAGE-1 is issued while tile j is computed.
+  constexpr int NSTAGE = 3;
+  constexpr int KPIECES = KBYTES / 1024 / NW, VPIECES = VBYTES / 1024 / NW;
+  static_assert(KPIECES * 1024 * NW == KBYTES && VPIECES * 1024 * NW == VBYTES, "tile must split into 1 KB pieces per wavefront");
+  auto dma16 = [&](const void* src, uint8_t* dst_uniform) {
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                     (__attribute__((address_space(3))) void*)dst_uniform, 16, 0, 0);
   };
-  auto store_tile = [&](uint8_t* stage) {
+  auto load_tile = [&](int j, uint8_t* stage) {
 #pragma unroll
-    for (int i = 0; i < KCH; i++) {
-      int c = i * NTHR + tid, n = c / CPR, cc = c % CPR;
-      if (KCHUNKS % NTHR == 0 || c < KCHUNKS)
-        *reinterpret_cast<v4i*>(stage + n * D + 16 * (cc ^ kswz<D>(n))) = kst[i];
+    for (int i = 0; i < KPIECES; i++) {
+      const int piece = i * NW + w;
+      const int sl = piece * 64 + lane, n = sl / CPR, cc = (sl % CPR) ^ kswz<D>(n);
+      const int row = min(j * BN + n, Lk - 1);
+      dma16(a.k + koff + (int64_t)row * a.k_sn + 16 * cc, stage + piece * 1024);
     }
+    const uint8_t* vsrc = vbase + (int64_t)j * VBYTES;
 #pragma unroll
-    for (int i = 0; i < VCH; i++)
-      if (VCHUNKS % NTHR == 0 || i * NTHR + tid < VCHUNKS)
-        *reinterpret_cast<v4i*>(stage + KBYTES + (i * NTHR + tid) * 16) = vst[i];
+    for (int i = 0; i < VPIECES; i++) {
+      const int piece = i * NW + w;
+      dma16(vsrc + piece * 1024 + lane * 16, stage + KBYTES + piece * 1024);
+    }
   };
 
   auto compute = [&](const uint8_t* stage, int j) {
@@ -210,7 +214,7 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
     }
     float sc[NT];
 #pragma unroll
-    for (int nt = 0; nt < NT; nt++) sc[nt] = qscale * ksp[min((n0 + 32 * nt) / a.blkk, nkblk - 1)];
+    for (int nt = 0; nt < NT; nt++) sc[nt] = qscale * ksp[min((n0 + 32 * nt) >> a.blkk_shift, nkblk - 1)];
 
     // ---- masking: only tiles that cross the diagonal or the end of the sequence ----
     const bool need_mask = (CAUSAL && (n0 + BN - 1 > row0)) || (n0 + BN > Lk);
@@ -304,16 +308,19 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
 
   // ---- main loop over KV tiles ----
   if (ntiles > 0) {
-    load_tile(0);
-    store_tile(smem);
-    __syncthreads();
+    uint8_t* s0 = smem;               // tile j
+    uint8_t* s1 = smem + STAGE;       // tile j+1
+    uint8_t* s2 = smem + 2 * STAGE;   // tile j+2 (being filled)
+    load_tile(0, s0);
+    if (ntiles > 1) load_tile(1, s1);
     for (int j = 0; j < ntiles; j++) {
-      uint8_t* cur = smem + (j & 1) * STAGE;
-      uint8_t* nxt = smem + ((j + 1) & 1) * STAGE;
-      if (j + 1 < ntiles) load_tile(j + 1);
-      if (j < wave_ntiles) compute(cur, j);
-      if (j + 1 < ntiles) store_tile(nxt);
-      __syncthreads();
+      // tile j must have landed: at most the loads of tile j+1 (issued one iteration ago) may be pending
+      if (j + 1 < ntiles) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(KPIECES + VPIECES) : "memory");
+      else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      lds_barrier();   // everyone's pieces of tile j are visible; everyone is done reading tile j-1
+      if (j + 2 < ntiles) load_tile(j + 2, s2);
+      if (j < wave_ntiles) compute(s0, j);
+      uint8_t* t = s0; s0 = s1; s1 = s2; s2 = t;
     }
   }
 
@@ -414,7 +421,7 @@ AttnConfig attn_config(int D, int pv, bool packed) {
 template <int D, int NW, int BN, int PV, bool CAUSAL>
 static hipError_t launch_one(const AttnArgs& a, int grid, hipStream_t st) {
   constexpr int VESZ = PV ? 1 : 2;
-  constexpr int smem = 2 * (BN * D + BN * D * VESZ);
+  constexpr int smem = 3 * (BN * D + BN * D * VESZ);
   auto kern = attn_kernel<D, NW, BN, PV, CAUSAL>;
   static bool attr_done = false;
   if (!attr_done) {
@@ -430,7 +437,7 @@ hipError_t launch_attn(const AttnArgs& a, int D, int pv, bool causal, int grid, 
   if (grid == 0) return hipSuccess;
 #define SAGE_ATTN(DD, PVV, BNN) (causal ? launch_one<DD, 8, BNN, PVV, true>(a, grid, st) : launch_one<DD, 8, BNN, PVV, false>(a, grid, st))
   if (D == 128) return pv ? SAGE_ATTN(128, 1, 128) : SAGE_ATTN(128, 0, 64);
-  return pv ? SAGE_ATTN(64, 1, 128) : SAGE_ATTN(64, 0, 64);
+  return pv ? SAGE_ATTN(64, 1, 128) : SAGE_ATTN(64, 0, 128);
 #undef SAGE_ATTN
 }
 

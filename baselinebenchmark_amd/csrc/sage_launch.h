@@ -49,7 +49,8 @@ struct AttnArgs {
   float* lse;
   int B, Hq, Hkv, Sq, Skv;
   int64_t q_sb, q_sh, q_sn, k_sb, k_sh, k_sn, o_sb, o_sh, o_sn;
-  int blkq, blkk;
+  int blkq, blkk;            // scale block sizes: powers of two (32, 64, 128)
+  int blkq_shift, blkk_shift;  // their log2
   int out_bf16;
   int nqt;  // q-tiles per sequence (fixed-length mode)
   // packed mode (cu_q != nullptr)
@@ -62,6 +63,7 @@ struct AttnArgs {
   const int32_t* tiles;
   int64_t qs_sh, ks_sh, panel_sh;
   int total_q;
+  int pp_split;  // 0: wavefront groups {0..NW/2-1 | NW/2..NW-1}; 1: even/odd wavefronts
 };
 
 struct AttnConfig { int nw, bn; };
