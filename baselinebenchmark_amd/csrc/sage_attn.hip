@@ -77,7 +77,7 @@ __device__ inline int kswz(int n) {
   return (n / RPB) % CPR;
 }
 
-template <int D, int NW, int BN, int PV, bool CAUSAL>
+template <int D, int NW, int BN, int PV, bool CAUSAL, bool MSUM>
 __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
   constexpr int BM = NW * 32;
   constexpr int NTHR = NW * 64;
@@ -167,6 +167,19 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
 #pragma unroll
     for (int i = 0; i < 16; i++) o[dt][i] = 0.f;
   float m_used = kMInit, lsum = 0.f;
+  // MSUM (FP8 mode when no LSE is requested): the row sums come out of the matrix pipe too.  A V^T operand of all ones (fp8 1.0 = 0x38)
+  // makes every row of one extra 32x32 output tile equal to sum_n P[n][m], i.e. the softmax
+  // denominator of query row m -- of the very fp8 values that multiply V.  That removes one VALU add
+  // per score (the VALU, not the MFMA pipe, is the busier unit of this kernel).  The sum of rounded
+  // values is the right denominator for O but costs LSE accuracy on rows with few keys, so kernels
+  // that return LSE keep the fp32 VALU sum.
+  v16f osum;
+#pragma unroll
+  for (int i = 0; i < 16; i++) osum[i] = 0.f;
+  v8i ones;
+#pragma unroll
+  for (int i = 0; i < 8; i++) ones[i] = 0x38383838;
+  asm volatile("" : "+v"(ones));
 
   // ---- tile loads: global memory -> LDS directly (no registers), 1 KB per wavefront instruction ----
   // Lane l of a wavefront writes LDS bytes [16*l, 16*l+16) of the 1 KB piece, so the K swizzle is
@@ -243,6 +256,10 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
       const float m_new = fmaxf(m_used, mloc);
       const float alpha = __builtin_amdgcn_exp2f(m_used - m_new);
       lsum *= alpha;
+      if constexpr (MSUM) {
+#pragma unroll
+        for (int i = 0; i < 16; i++) osum[i] *= alpha;
+      }
 #pragma unroll
       for (int dt = 0; dt < DTN; dt++)
 #pragma unroll
@@ -260,11 +277,13 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
 #pragma unroll
         for (int r = 0; r < 16; r++) {
           p[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(as_f(acc[nt][r]), sc[nt], c));
-          lsum += p[r];
+          if constexpr (!MSUM) lsum += p[r];
         }
 #pragma unroll
         for (int q4 = 0; q4 < 4; q4++) {
-          int d0 = __builtin_amdgcn_cvt_pk_fp8_f32(p[4 * q4], p[4 * q4 + 1], 0, false);
+          // both halves of the dword get written, so the 'old' operand is a don't-care: reuse a dead
+          // accumulator register instead of materialising a zero
+          int d0 = __builtin_amdgcn_cvt_pk_fp8_f32(p[4 * q4], p[4 * q4 + 1], acc[nt][4 * q4], false);
           pk[nt][q4] = __builtin_amdgcn_cvt_pk_fp8_f32(p[4 * q4 + 2], p[4 * q4 + 3], d0, true);
         }
       }
@@ -274,6 +293,7 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
         v8i pb;
 #pragma unroll
         for (int i = 0; i < 4; i++) { pb[i] = pk[2 * kk][i]; pb[4 + i] = pk[2 * kk + 1][i]; }
+        if constexpr (MSUM) osum = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ones, pb, osum, 0, 0, 0, 0, 0, 0);
 #pragma unroll
         for (int dt = 0; dt < DTN; dt++) {
           const uint8_t* vp0 = vbuf + (((kk * DTN + dt) * 2) * 64 + lane) * 16;
@@ -325,7 +345,8 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
   }
 
   // ---- epilogue: O = O^T / l (* v_scale), LSE2 = m + log2(l) ----
-  lsum = xchg32_sum(lsum);
+  if constexpr (MSUM) lsum = osum[0];   // already the full row sum (the MFMA contracts over both lane halves)
+  else lsum = xchg32_sum(lsum);
   const float inv = lsum > 0.f ? 1.0f / lsum : 0.f;
   if (my_row < Lq) {
     if (a.lse && h == 0) a.lse[lseoff + my_row] = lsum > 0.f ? m_used + __builtin_amdgcn_logf(lsum) - PSHIFT : kNegInf;
@@ -418,11 +439,11 @@ AttnConfig attn_config(int D, int pv, bool packed) {
   return c;
 }
 
-template <int D, int NW, int BN, int PV, bool CAUSAL>
+template <int D, int NW, int BN, int PV, bool CAUSAL, bool MSUM>
 static hipError_t launch_one(const AttnArgs& a, int grid, hipStream_t st) {
   constexpr int VESZ = PV ? 1 : 2;
   constexpr int smem = 3 * (BN * D + BN * D * VESZ);
-  auto kern = attn_kernel<D, NW, BN, PV, CAUSAL>;
+  auto kern = attn_kernel<D, NW, BN, PV, CAUSAL, MSUM>;
   static bool attr_done = false;
   if (!attr_done) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
@@ -435,9 +456,10 @@ static hipError_t launch_one(const AttnArgs& a, int grid, hipStream_t st) {
 
 hipError_t launch_attn(const AttnArgs& a, int D, int pv, bool causal, int grid, hipStream_t st) {
   if (grid == 0) return hipSuccess;
-#define SAGE_ATTN(DD, PVV, BNN) (causal ? launch_one<DD, 8, BNN, PVV, true>(a, grid, st) : launch_one<DD, 8, BNN, PVV, false>(a, grid, st))
-  if (D == 128) return pv ? SAGE_ATTN(128, 1, 128) : SAGE_ATTN(128, 0, 64);
-  return pv ? SAGE_ATTN(64, 1, 128) : SAGE_ATTN(64, 0, 128);
+  const bool msum = pv && a.lse == nullptr;   // row sums on the matrix pipe unless LSE is wanted
+#define SAGE_ATTN(DD, PVV, BNN, MS) (causal ? launch_one<DD, 8, BNN, PVV, true, MS>(a, grid, st) : launch_one<DD, 8, BNN, PVV, false, MS>(a, grid, st))
+  if (D == 128) return pv ? (msum ? SAGE_ATTN(128, 1, 128, true) : SAGE_ATTN(128, 1, 128, false)) : SAGE_ATTN(128, 0, 64, false);
+  return pv ? (msum ? SAGE_ATTN(64, 1, 128, true) : SAGE_ATTN(64, 1, 128, false)) : SAGE_ATTN(64, 0, 128, false);
 #undef SAGE_ATTN
 }
 

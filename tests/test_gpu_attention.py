@@ -199,8 +199,15 @@ def test_long_sequence_properties_full_size_head():
                                  attn_mask=(torch.arange(S)[None, :] <= torch.arange(S - T, S)[:, None])[None, None])
     assert oa.metrics(o[:, :, S - T:], ref_t)["cosine"] >= 0.999
     # linearity in V: doubling V doubles the output (per-channel scales absorb the factor exactly)
-    out2, _ = sa.forward(qi, ki, vg * 2, qs, ks, output_dtype=torch.bfloat16, BLKQ=64, BLKK=128, is_causal=True, pv_mode="fp8")
+    out2, _ = sa.forward(qi, ki, vg * 2, qs, ks, output_dtype=torch.bfloat16, return_lse=True, BLKQ=64, BLKK=128,
+                         is_causal=True, pv_mode="fp8")
     assert torch.equal(out2.cpu().float(), o * 2)
+    # without LSE the row sums are taken on the matrix pipe from the fp8-rounded probabilities: same answer
+    # up to that rounding, and itself exactly linear in V
+    out3, _ = sa.forward(qi, ki, vg, qs, ks, output_dtype=torch.bfloat16, BLKQ=64, BLKK=128, is_causal=True, pv_mode="fp8")
+    out4, _ = sa.forward(qi, ki, vg * 2, qs, ks, output_dtype=torch.bfloat16, BLKQ=64, BLKK=128, is_causal=True, pv_mode="fp8")
+    assert torch.equal(out4.cpu().float(), out3.cpu().float() * 2)
+    assert oa.metrics(out3.cpu().float(), o)["cosine"] >= 0.9995
 
 
 def test_lse_is_empty_unless_requested():
