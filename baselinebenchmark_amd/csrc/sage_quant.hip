@@ -109,14 +109,13 @@ __global__ void __launch_bounds__(256) quant_int8_kernel(QuantArgs a) {
         x = x * a.mult;
         float z;
         if (fast) {
+          // For |x| so small that the residual of the correction step is subnormal the quotient is
+          // below 1e-13 in magnitude (scale >= 1e-12): whatever its last bits, it rounds to 0.
           z = div_by_uniform(x, scale, rcp);
-          // tiny |x| could make the residual subnormal; its quotient is below 1e-13 in magnitude
-          // (scale >= 1e-12) and rounds to 0 whatever its sign
-          if (fabsf(x) < 1.0e-25f) z = 0.f;
         } else {
           z = x / scale;
         }
-        z = (z >= 0.f) ? z + 0.5f : z - 0.5f;
+        z = z + __builtin_copysignf(0.5f, z);   // +0.5 for z >= 0 (incl. -0: -0.5 + -0 = -0.5 -> 0), else -0.5
         int q = (int)z;  // truncation toward zero
         packed[i >> 2] |= (uint32_t)(q & 0xff) << (8 * (i & 3));
       }
