@@ -29,9 +29,10 @@ __device__ inline float div_by_uniform(float x, float s, float r) {
 
 // One workgroup (256 lanes) quantises one [blk, D] tile held entirely in registers:
 // pass 1 converts and reduces |x| to the tile maximum, pass 2 divides and rounds.
+// A lane owns 16 consecutive channels of a row (two 128-bit loads, one 128-bit store).
 template <int DT, int D>
 __global__ void __launch_bounds__(256) quant_int8_kernel(QuantArgs a) {
-  constexpr int TPR = D / 8;        // lanes per row (8 elements = 16 bytes each)
+  constexpr int TPR = D / 16;       // lanes per row
   constexpr int RPP = 256 / TPR;    // rows per pass
   constexpr int MAXP = 128 / RPP;   // passes for the largest tile (128 rows)
   const int blkid = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
@@ -55,31 +56,34 @@ __global__ void __launch_bounds__(256) quant_int8_kernel(QuantArgs a) {
   if (n0 >= L) return;
   const int rows = min(a.blk, L - n0);
 
-  float kmv[8];
+  float kmv[16];
   const bool has_km = a.km != nullptr;
   if (has_km) {
-    uint4 raw = *reinterpret_cast<const uint4*>(a.km + (int64_t)b * a.km_sb + (int64_t)h * a.km_sh + tc * 8);
-    const u16* p = reinterpret_cast<const u16*>(&raw);
+    const uint4* kp = reinterpret_cast<const uint4*>(a.km + (int64_t)b * a.km_sb + (int64_t)h * a.km_sh + tc * 16);
+    uint4 raw2[2] = {kp[0], kp[1]};
+    const u16* p = reinterpret_cast<const u16*>(raw2);
 #pragma unroll
-    for (int i = 0; i < 8; i++) kmv[i] = to_f32<DT>(p[i]);
+    for (int i = 0; i < 16; i++) kmv[i] = to_f32<DT>(p[i]);
   }
+  auto value = [&](u16 bits, int i) {   // the fp32 value that is quantised
+    float x = to_f32<DT>(bits);
+    if (has_km) x = to_f32<DT>(from_f32<DT>(x - kmv[i]));
+    return x * a.mult;
+  };
 
-  uint4 raw[MAXP];
+  uint4 raw[MAXP][2];
   float amax = 0.f;
 #pragma unroll
   for (int p = 0; p < MAXP; p++) {
     int r = p * RPP + tr;
-    raw[p] = make_uint4(0, 0, 0, 0);
+    raw[p][0] = raw[p][1] = make_uint4(0, 0, 0, 0);
     if (r < rows) {
-      raw[p] = *reinterpret_cast<const uint4*>(a.x + xbase + (int64_t)(n0 + r) * a.x_sn + tc * 8);
-      const u16* e = reinterpret_cast<const u16*>(&raw[p]);
+      const uint4* src = reinterpret_cast<const uint4*>(a.x + xbase + (int64_t)(n0 + r) * a.x_sn + tc * 16);
+      raw[p][0] = src[0];
+      raw[p][1] = src[1];
+      const u16* e = reinterpret_cast<const u16*>(raw[p]);
 #pragma unroll
-      for (int i = 0; i < 8; i++) {
-        float x = to_f32<DT>(e[i]);
-        if (has_km) x = to_f32<DT>(from_f32<DT>(x - kmv[i]));
-        x = x * a.mult;
-        amax = fmaxf(amax, fabsf(x));
-      }
+      for (int i = 0; i < 16; i++) amax = fmaxf(amax, fabsf(value(e[i], i)));
     }
   }
   __shared__ float wmax[4];
@@ -91,8 +95,8 @@ __global__ void __launch_bounds__(256) quant_int8_kernel(QuantArgs a) {
   if (tid == 0) a.scale[sidx] = scale;
 
   const float rcp = 1.0f / scale;
-  // The fast correction-step division needs: significand of scale not all ones, and scale, rcp
-  // and every quotient comfortably normal.  |quotient| <= 127.5, scale >= 1e-12.
+  // The fast correction-step division needs: significand of scale not all ones, and scale and rcp
+  // comfortably normal.  |quotient| <= 127.5, scale >= 1e-12.
   const uint32_t sbits = __builtin_bit_cast(uint32_t, scale);
   const bool fast = ((sbits & 0x7fffffu) != 0x7fffffu) && scale < 1.0e30f;
 
@@ -100,13 +104,11 @@ __global__ void __launch_bounds__(256) quant_int8_kernel(QuantArgs a) {
   for (int p = 0; p < MAXP; p++) {
     int r = p * RPP + tr;
     if (r < rows) {
-      const u16* e = reinterpret_cast<const u16*>(&raw[p]);
-      uint32_t packed[2] = {0, 0};
+      const u16* e = reinterpret_cast<const u16*>(raw[p]);
+      uint32_t packed[4] = {0, 0, 0, 0};
 #pragma unroll
-      for (int i = 0; i < 8; i++) {
-        float x = to_f32<DT>(e[i]);
-        if (has_km) x = to_f32<DT>(from_f32<DT>(x - kmv[i]));
-        x = x * a.mult;
+      for (int i = 0; i < 16; i++) {
+        const float x = value(e[i], i);
         float z;
         if (fast) {
           // For |x| so small that the residual of the correction step is subnormal the quotient is
@@ -119,7 +121,7 @@ __global__ void __launch_bounds__(256) quant_int8_kernel(QuantArgs a) {
         int q = (int)z;  // truncation toward zero
         packed[i >> 2] |= (uint32_t)(q & 0xff) << (8 * (i & 3));
       }
-      *reinterpret_cast<uint2*>(a.out + obase + (int64_t)(n0 + r) * a.o_sn + tc * 8) = make_uint2(packed[0], packed[1]);
+      *reinterpret_cast<uint4*>(a.out + obase + (int64_t)(n0 + r) * a.o_sn + tc * 16) = make_uint4(packed[0], packed[1], packed[2], packed[3]);
     }
   }
 }

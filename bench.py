@@ -106,6 +106,9 @@ def main():
     ap.add_argument("--workload", default="c2", choices=["c0", "c1", "c2", "c3", "c4"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=20.0)
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run three 512 MiB device-to-device copies (a kernel of known traffic, used to scale "
+                         "the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this path is built and measured on a single MI355X "
@@ -155,6 +158,12 @@ def main():
                    "effective_ops": w.ops, "frac_of_mfma_peak_end_to_end": round(value / peak, 4)},
         "roofline": roofline,
     }
+    if args.copy_calibration:
+        x = torch.empty(128 * 1024 * 1024, device="cuda", dtype=torch.int32)
+        y = torch.empty_like(x)
+        for _ in range(3):
+            y.copy_(x)
+        torch.cuda.synchronize()
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(args.workload if args.workload != "c4" else "c2", args.cpu_seconds)
     print(json.dumps(out))
