@@ -212,10 +212,18 @@ __global__ void vscale_finalize_kernel(const float* partial, float* vscale, int 
 
 template <int DT, int D, int PV>
 __global__ void __launch_bounds__(256) prep_v_kernel(PrepVArgs a) {
-  constexpr int TPR = D / 8, RPP = 256 / TPR, NP = kPanelRows / RPP;
+  // A lane converts 4 consecutive rows x 8 consecutive channels at a time, so that the 4 row values of
+  // a channel pack into one dword (fp8) or two (fp16): exactly the (b = 0..3) group of the panel
+  // order.  They are staged in LDS as T[channel][row quad] and read back in panel order.
+  constexpr int TPR = D / 8, RPP = 256 / TPR;   // lanes per row, row quads handled per pass
+  constexpr int NQ = kPanelRows / 4;            // 32 row quads per panel
+  constexpr int QPT = NQ / RPP;                 // passes
   constexpr int ESZ = (PV == 1) ? 1 : 2;
+  constexpr int QW = ESZ;                       // dwords per (channel, row quad)
+  constexpr int TS = NQ * QW + 1;               // dword stride of a channel in LDS (padded)
   constexpr int PANEL_BYTES = kPanelRows * D * ESZ;
-  __shared__ __attribute__((aligned(16))) uint8_t stage[PANEL_BYTES];
+  constexpr int DTN = D / 32;
+  __shared__ uint32_t T[D * TS];
   const int pidx = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
   const int tid = threadIdx.x, tr = tid / TPR, tc = tid % TPR;
   int L = a.L;
@@ -231,36 +239,69 @@ __global__ void __launch_bounds__(256) prep_v_kernel(PrepVArgs a) {
   }
   const int n0 = pidx * kPanelRows;
   if (n0 >= L) return;
-  float sc[8];
+  float sc[8], rc[8];
+  bool fast = true;
   if constexpr (PV == 1) {
 #pragma unroll
-    for (int i = 0; i < 8; i++) sc[i] = a.vscale[((int64_t)b * a.H + h) * D + tc * 8 + i];
+    for (int i = 0; i < 8; i++) {
+      sc[i] = a.vscale[((int64_t)b * a.H + h) * D + tc * 8 + i];
+      rc[i] = 1.0f / sc[i];
+      fast = fast && ((__builtin_bit_cast(uint32_t, sc[i]) & 0x7fffffu) != 0x7fffffu) && sc[i] < 1.0e30f;
+    }
+    fast = __builtin_amdgcn_ballot_w64(!fast) == 0;   // the correction-step division for the whole wavefront, or not at all
   }
 #pragma unroll
-  for (int p = 0; p < NP; p++) {
-    int r = p * RPP + tr;
-    uint4 raw = make_uint4(0, 0, 0, 0);
-    if (n0 + r < L) raw = *reinterpret_cast<const uint4*>(a.v + vbase + (int64_t)(n0 + r) * a.v_sn + tc * 8);
-    const u16* e = reinterpret_cast<const u16*>(&raw);
+  for (int qq = 0; qq < QPT; qq++) {
+    const int quad = qq * RPP + tr;
+    uint4 raw[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      const int r = n0 + 4 * quad + j;
+      raw[j] = make_uint4(0, 0, 0, 0);
+      if (r < L) raw[j] = *reinterpret_cast<const uint4*>(a.v + vbase + (int64_t)r * a.v_sn + tc * 8);
+    }
 #pragma unroll
     for (int i = 0; i < 8; i++) {
-      float x = to_f32<DT>(e[i]);
-      int d = tc * 8 + i;
+      float x[4];
+#pragma unroll
+      for (int j = 0; j < 4; j++) x[j] = to_f32<DT>(reinterpret_cast<const u16*>(&raw[j])[i]);
+      uint32_t* dst = &T[(tc * 8 + i) * TS + quad * QW];
       if constexpr (PV == 1) {
-        float z = x / sc[i];
-        z = fminf(fmaxf(z, -448.f), 448.f);
-        int pk = __builtin_amdgcn_cvt_pk_fp8_f32(z, z, 0, false);
-        stage[panel_index_fp8(r, d, D)] = (uint8_t)(pk & 0xff);
+        float z[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          z[j] = fast ? div_by_uniform(x[j], sc[i], rc[i]) : x[j] / sc[i];
+          z[j] = fminf(fmaxf(z[j], -448.f), 448.f);
+        }
+        int pk = __builtin_amdgcn_cvt_pk_fp8_f32(z[0], z[1], 0, false);
+        pk = __builtin_amdgcn_cvt_pk_fp8_f32(z[2], z[3], pk, true);
+        dst[0] = (uint32_t)pk;
       } else {
-        reinterpret_cast<u16*>(stage)[panel_index_fp16(r, d, D)] = f32_to_f16(x);
+        dst[0] = (uint32_t)f32_to_f16(x[0]) | ((uint32_t)f32_to_f16(x[1]) << 16);
+        dst[1] = (uint32_t)f32_to_f16(x[2]) | ((uint32_t)f32_to_f16(x[3]) << 16);
       }
     }
   }
   __syncthreads();
-  const uint4* src = reinterpret_cast<const uint4*>(stage);
-  uint4* dst = reinterpret_cast<uint4*>(a.panels + pbase);
+  uint4* out = reinterpret_cast<uint4*>(a.panels + pbase);
 #pragma unroll
-  for (int i = 0; i < PANEL_BYTES / 16 / 256; i++) dst[i * 256 + tid] = src[i * 256 + tid];
+  for (int i = 0; i < PANEL_BYTES / 16 / 256; i++) {
+    const int c = i * 256 + tid;           // 16-byte chunk of the panel
+    const int lane = c & 63, hh = lane >> 5, d_lo = lane & 31;
+    uint4 v;
+    if constexpr (PV == 1) {
+      // c = ((ks*DTN + dt)*2 + half)*64 + lane ; bytes 4a+b <-> row 64ks + 32half + 8a + 4h + b
+      const int half = (c >> 6) & 1, dt = (c >> 7) % DTN, ks = (c >> 7) / DTN;
+      const uint32_t* src = &T[(32 * dt + d_lo) * TS + 16 * ks + 8 * half + hh];
+      v = make_uint4(src[0], src[2], src[4], src[6]);
+    } else {
+      // c = (ks16*DTN + dt)*64 + lane ; elements 4a+b <-> row 16ks16 + 8a + 4h + b
+      const int dt = (c >> 6) % DTN, ks16 = (c >> 6) / DTN;
+      const uint32_t* src = &T[(32 * dt + d_lo) * TS + (4 * ks16 + hh) * 2];
+      v = make_uint4(src[0], src[1], src[4], src[5]);
+    }
+    out[c] = v;
+  }
 }
 
 // ---------------------------------------------------------------------------------------------
