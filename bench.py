@@ -29,6 +29,12 @@ PEAK_INT8_FP8 = 5033.2   # MI355X dense INT8 / FP8 MFMA peak, TOP/s (256 CUs x 2
 PEAK_FP16 = 2516.6       # dense FP16 MFMA peak, TFLOP/s
 
 
+# HBM-side bytes per launch of the attention kernel, from the committed rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# runs on this same command (profiles/attn_kernel_c2_pmc.md): (1 180 240 + 262 148) counter units x 2.0 (the factor the
+# same counters read for a 512 MiB device copy) x 1 KiB.  Measured for config 2 only.
+TRAFFIC_BYTES = {"c2": (1180240 + 262148) * 2.0 * 1024}
+
+
 def blended_peak(pv: str) -> float:
     """FP8 P.V: both GEMMs run at the INT8/FP8 rate.  FP16 P.V: half of the ops run at the FP16 rate."""
     if pv == "fp8":
@@ -146,7 +152,7 @@ def main():
     if kms is not None:
         achieved = w.ops / (kms * 1e-3) / 1e12
         roofline = {"bound": "mfma", "achieved": round(achieved, 1), "peak": round(peak, 1), "unit": "TFLOP/s",
-                    "frac": round(achieved / peak, 4), "traffic": None,
+                    "frac": round(achieved / peak, 4), "traffic": TRAFFIC_BYTES.get(args.workload),
                     "kernel": "sage::attn_kernel", "kernel_ms": round(kms, 4),
                     "note": "algorithmic ops = 4*B*Hq*Sq*Skv*D*(1/2 causal) per launch / HIP-event average launch time"}
     out = {
