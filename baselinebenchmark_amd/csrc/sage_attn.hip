@@ -139,6 +139,9 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
     vbase = a.vp + ((int64_t)b * a.Hkv + kvh) * ((Lk + kPanelRows - 1) / kPanelRows) * PANEL_BYTES;
   }
   nkblk = (Lk + a.blkk - 1) / a.blkk;
+  // The K scales are read through the scalar cache (constant address space): a vector load would sit
+  // in the same in-order counter as the tile loads in flight and make every tile wait for them.
+  const __attribute__((address_space(4))) float* ksc = (const __attribute__((address_space(4))) float*)ksp;
 
   const int row0 = qt * BM + w * 32;   // first query row of this wavefront
   const int my_row = row0 + m;
@@ -213,21 +216,35 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
     const uint8_t* kbuf = stage;
     const uint8_t* vbuf = stage + KBYTES;
     // ---- S^T = K . Q^T (int8 -> int32 on the biased accumulators) ----
+    // K fragments run KPF MFMAs ahead of their use so that no MFMA waits for the LDS read issued
+    // just before it; the k-step is the outer index so that consecutive MFMAs hit different accumulators.
     v16i acc[NT];
+    {
+      constexpr int NF = NT * KS, KPF = 4;
+      auto kfrag = [&](int i) {
+        const int nt = i % NT, ks = i / NT, n = 32 * nt + m;
+        return *reinterpret_cast<const v4i*>(kbuf + n * D + 16 * ((2 * ks + h) ^ kswz<D>(n)));
+      };
+      v4i kf[NF];
 #pragma unroll
-    for (int nt = 0; nt < NT; nt++) {
-      const int n = 32 * nt + m;
-      const uint8_t* rowp = kbuf + n * D;
-      const int sw = kswz<D>(n);
+      for (int i = 0; i < KPF; i++) kf[i] = kfrag(i);
 #pragma unroll
-      for (int ks = 0; ks < KS; ks++) {
-        v4i ka = *reinterpret_cast<const v4i*>(rowp + 16 * ((2 * ks + h) ^ sw));
-        acc[nt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ka, qreg[ks], ks == 0 ? bias : acc[nt], 0, 0, 0);
+      for (int i = 0; i < NF; i++) {
+        if (i + KPF < NF) kf[i + KPF] = kfrag(i + KPF);
+        const int nt = i % NT, ks = i / NT;
+        acc[nt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf[i], qreg[ks], ks == 0 ? bias : acc[nt], 0, 0, 0);
       }
+      __builtin_amdgcn_sched_group_barrier(0x100, KPF, 0);
+#pragma unroll
+      for (int i = 0; i < NF - KPF; i++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, KPF, 0);
     }
     float sc[NT];
 #pragma unroll
-    for (int nt = 0; nt < NT; nt++) sc[nt] = qscale * ksp[min((n0 + 32 * nt) >> a.blkk_shift, nkblk - 1)];
+    for (int nt = 0; nt < NT; nt++) sc[nt] = qscale * ksc[min((n0 + 32 * nt) >> a.blkk_shift, nkblk - 1)];
 
     // ---- masking: only tiles that cross the diagonal or the end of the sequence ----
     const bool need_mask = (CAUSAL && (n0 + BN - 1 > row0)) || (n0 + BN > Lk);
@@ -288,19 +305,28 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
         }
       }
       // ---- O^T += V^T . P^T ----
-#pragma unroll
-      for (int kk = 0; kk < BN / 64; kk++) {
-        v8i pb;
-#pragma unroll
-        for (int i = 0; i < 4; i++) { pb[i] = pk[2 * kk][i]; pb[4 + i] = pk[2 * kk + 1][i]; }
-        if constexpr (MSUM) osum = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ones, pb, osum, 0, 0, 0, 0, 0, 0);
-#pragma unroll
-        for (int dt = 0; dt < DTN; dt++) {
-          const uint8_t* vp0 = vbuf + (((kk * DTN + dt) * 2) * 64 + lane) * 16;
+      {
+        constexpr int NV = (BN / 64) * DTN, VPF = 2;
+        auto vfrag = [&](int i) {
+          const uint8_t* vp0 = vbuf + ((i * 2) * 64 + lane) * 16;
           v4i lo = *reinterpret_cast<const v4i*>(vp0);
           v4i hi = *reinterpret_cast<const v4i*>(vp0 + 64 * 16);
-          v8i va = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-          o[dt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(va, pb, o[dt], 0, 0, 0, 0, 0, 0);
+          return v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        };
+        v8i vf[NV];
+#pragma unroll
+        for (int i = 0; i < VPF; i++) vf[i] = vfrag(i);
+#pragma unroll
+        for (int i = 0; i < NV; i++) {
+          const int kk = i / DTN, dt = i % DTN;
+          if (i + VPF < NV) vf[i + VPF] = vfrag(i + VPF);
+          v8i pb;
+#pragma unroll
+          for (int e = 0; e < 4; e++) { pb[e] = pk[2 * kk][e]; pb[4 + e] = pk[2 * kk + 1][e]; }
+          if constexpr (MSUM) {
+            if (dt == 0) osum = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ones, pb, osum, 0, 0, 0, 0, 0, 0);
+          }
+          o[dt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vf[i], pb, o[dt], 0, 0, 0, 0, 0, 0);
         }
       }
     } else {
