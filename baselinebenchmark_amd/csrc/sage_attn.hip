@@ -24,8 +24,17 @@
 //   * K/V tiles go global -> registers -> LDS, double buffered, one barrier per KV tile.
 #include "sage_launch.h"
 #include <cstdlib>
+#ifndef SAGE_GSH
+#define SAGE_GSH 2
+#endif
 
 namespace sage {
+#ifdef SAGE_TIMING
+__device__ long long g_timing[8 * 8];
+#define TICK(i) do { long long t_ = clock64(); tacc[i] += t_ - tlast; tlast = t_; } while (0)
+#else
+#define TICK(i)
+#endif
 
 
 constexpr float kBiasF = 12582912.0f;     // 1.5 * 2^23
@@ -79,6 +88,7 @@ __device__ inline int kswz(int n) {
 
 template <int D, int NW, int BN, int PV, bool CAUSAL, bool MSUM>
 __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
+  constexpr int GSH = SAGE_GSH;   // which bit of the wavefront index picks the group
   constexpr int BM = NW * 32;
   constexpr int NTHR = NW * 64;
   constexpr int KS = D / 32;   // contraction steps of S^T
@@ -187,38 +197,60 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
   // ---- tile loads: global memory -> LDS directly (no registers), 1 KB per wavefront instruction ----
   // Lane l of a wavefront writes LDS bytes [16*l, 16*l+16) of the 1 KB piece, so the K swizzle is
   // applied on the global side: the lane fetches the 16-byte chunk that belongs in its slot.
-  // Stages form a ring of NSTAGE tiles; the load of tile j+NSTAGE-1 is issued while tile j is computed.
-  constexpr int NSTAGE = 3;
+  // K tiles and V tiles each alternate between two LDS slots.
   constexpr int KPIECES = KBYTES / 1024 / NW, VPIECES = VBYTES / 1024 / NW;
   static_assert(KPIECES * 1024 * NW == KBYTES && VPIECES * 1024 * NW == VBYTES, "tile must split into 1 KB pieces per wavefront");
-  auto dma16 = [&](const void* src, uint8_t* dst_uniform) {
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                     (__attribute__((address_space(3))) void*)dst_uniform, 16, 0, 0);
+  // The buffer form of the LDS load is used on purpose: the compiler treats the global form as a flat
+  // access that may touch LDS and then drains every counter at each LDS read while one is in flight.
+  const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc((void*)(a.k + koff), 0, 0x7fffffff, 0x00020000);
+  const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc((void*)vbase, 0, 0x7fffffff, 0x00020000);
+  auto dma16 = [&](__amdgpu_buffer_rsrc_t rsrc, int lane_offset, int uniform_offset, uint8_t* dst_uniform) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)dst_uniform, 16, lane_offset, uniform_offset, 0, 0);
   };
-  auto load_tile = [&](int j, uint8_t* stage) {
+  auto kslot = [&](int j) { return smem + (j & 1) * KBYTES; };
+  auto vslot = [&](int j) { return smem + 2 * KBYTES + (j & 1) * VBYTES; };
+  // Per-lane byte offsets of this wavefront's pieces inside a tile are loop invariant; the tile index
+  // only adds a uniform term.  Rows past the end of the sequence (last tile only) are clamped.
+  int koffv[KPIECES], voffv[VPIECES];
 #pragma unroll
-    for (int i = 0; i < KPIECES; i++) {
-      const int piece = i * NW + w;
-      const int sl = piece * 64 + lane, n = sl / CPR, cc = (sl % CPR) ^ kswz<D>(n);
-      const int row = min(j * BN + n, Lk - 1);
-      dma16(a.k + koff + (int64_t)row * a.k_sn + 16 * cc, stage + piece * 1024);
-    }
-    const uint8_t* vsrc = vbase + (int64_t)j * VBYTES;
+  for (int i = 0; i < KPIECES; i++) {
+    const int sl = (i * NW + w) * 64 + lane, n = sl / CPR, cc = (sl % CPR) ^ kswz<D>(n);
+    koffv[i] = n * (int)a.k_sn + 16 * cc;
+  }
 #pragma unroll
-    for (int i = 0; i < VPIECES; i++) {
-      const int piece = i * NW + w;
-      dma16(vsrc + piece * 1024 + lane * 16, stage + KBYTES + piece * 1024);
+  for (int i = 0; i < VPIECES; i++) voffv[i] = (i * NW + w) * 1024 + lane * 16;
+  const int ktile_bytes = BN * (int)a.k_sn;
+  auto load_k = [&](int j) {
+    uint8_t* dst = kslot(j);
+    if (j * BN + BN <= Lk) {
+#pragma unroll
+      for (int i = 0; i < KPIECES; i++) dma16(krsrc, koffv[i], j * ktile_bytes, dst + (i * NW + w) * 1024);
+    } else {
+#pragma unroll
+      for (int i = 0; i < KPIECES; i++) {
+        const int sl = (i * NW + w) * 64 + lane, n = sl / CPR, cc = (sl % CPR) ^ kswz<D>(n);
+        dma16(krsrc, min(j * BN + n, Lk - 1) * (int)a.k_sn + 16 * cc, 0, dst + (i * NW + w) * 1024);
+      }
     }
+  };
+  auto load_v = [&](int j) {
+    uint8_t* dst = vslot(j);
+#pragma unroll
+    for (int i = 0; i < VPIECES; i++) dma16(vrsrc, voffv[i], j * VBYTES, dst + (i * NW + w) * 1024);
   };
 
-  auto compute = [&](const uint8_t* stage, int j) {
-    const int n0 = j * BN;
-    const uint8_t* kbuf = stage;
-    const uint8_t* vbuf = stage + KBYTES;
-    // ---- S^T = K . Q^T (int8 -> int32 on the biased accumulators) ----
+  // State that crosses phases: the raw scores of the tile in flight, its row maximum and scales, and
+  // the probabilities packed as the B operand of the second MFMA.
+  v16i acc[NT];
+  float sc[NT];
+  float mloc = kNegInf;
+  v8h ph[NT][2];      // fp16 mode
+
+  // ---- S^T = K . Q^T (int8 -> int32 on the biased accumulators), then mask and row maximum ----
+  auto qk = [&](int j) {
+    const uint8_t* kbuf = kslot(j);
     // K fragments run KPF MFMAs ahead of their use so that no MFMA waits for the LDS read issued
     // just before it; the k-step is the outer index so that consecutive MFMAs hit different accumulators.
-    v16i acc[NT];
     {
       constexpr int NF = NT * KS, KPF = 4;
       auto kfrag = [&](int i) {
@@ -242,10 +274,16 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
       }
       __builtin_amdgcn_sched_group_barrier(0x008, KPF, 0);
     }
-    float sc[NT];
+  };
+  // q_scale * k_scale of the 32-key groups of tile j.  Fetched during the vector-ALU phase: a scalar
+  // load in flight while K/V fragments are being read would force every LDS wait to drain the queue.
+  auto load_scales = [&](int j) {
 #pragma unroll
-    for (int nt = 0; nt < NT; nt++) sc[nt] = qscale * ksc[min((n0 + 32 * nt) >> a.blkk_shift, nkblk - 1)];
+    for (int nt = 0; nt < NT; nt++) sc[nt] = qscale * ksc[min((j * BN + 32 * nt) >> a.blkk_shift, nkblk - 1)];
+  };
 
+  auto rowmax = [&](int j) {
+    const int n0 = j * BN;
     // ---- masking: only tiles that cross the diagonal or the end of the sequence ----
     const bool need_mask = (CAUSAL && (n0 + BN - 1 > row0)) || (n0 + BN > Lk);
     if (need_mask) {
@@ -254,11 +292,15 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
       for (int nt = 0; nt < NT; nt++)
 #pragma unroll
         for (int r = 0; r < 16; r++)
-          if (32 * nt + 8 * (r / 4) + (r % 4) > lim) acc[nt][r] = as_i(kNegInf);
+        {
+          // branch-free select on the sign of (lim - index): compare-and-select would hold 64 lane masks
+          // in scalar registers at once
+          const int gone = (lim - (32 * nt + 8 * (r / 4) + (r % 4))) >> 31;
+          acc[nt][r] = (acc[nt][r] & ~gone) | (as_i(kNegInf) & gone);
+        }
     }
-
     // ---- row maximum of this tile, in score units ----
-    float mloc = kNegInf;
+    mloc = kNegInf;
 #pragma unroll
     for (int nt = 0; nt < NT; nt++) {
       float mx = as_f(acc[nt][0]);
@@ -266,11 +308,14 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
       for (int r = 1; r < 16; r++) mx = fmaxf(mx, as_f(acc[nt][r]));
       mloc = fmaxf(mloc, __builtin_fmaf(mx, sc[nt], -kBiasF * sc[nt]));
     }
-    mloc = xchg32_max(mloc);
+  };
 
-    // ---- lazy rescale: move the reference maximum only when it grew by more than TAU ----
-    if (__builtin_amdgcn_ballot_w64(mloc > m_used + TAU) != 0) {
-      const float m_new = fmaxf(m_used, mloc);
+  // ---- online softmax of the tile whose scores are in acc: pure VALU work ----
+  auto softmax = [&](int j) {
+    const float mall = xchg32_max(mloc);
+    // lazy rescale: move the reference maximum only when it grew by more than TAU
+    if (__builtin_amdgcn_ballot_w64(mall > m_used + TAU) != 0) {
+      const float m_new = fmaxf(m_used, mall);
       const float alpha = __builtin_amdgcn_exp2f(m_used - m_new);
       lsum *= alpha;
       if constexpr (MSUM) {
@@ -283,10 +328,8 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
         for (int i = 0; i < 16; i++) o[dt][i] *= alpha;
       m_used = m_new;
     }
-
-    // ---- P = exp2(S - m) * 2^PSHIFT, packed straight into the B operand of the second MFMA ----
+    // P = exp2(S - m) * 2^PSHIFT, packed straight into the B operand of the second MFMA
     if constexpr (PV == 1) {
-      v4i pk[NT];
 #pragma unroll
       for (int nt = 0; nt < NT; nt++) {
         const float c = __builtin_fmaf(-kBiasF, sc[nt], PSHIFT - m_used);
@@ -299,38 +342,13 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
 #pragma unroll
         for (int q4 = 0; q4 < 4; q4++) {
           // both halves of the dword get written, so the 'old' operand is a don't-care: reuse a dead
-          // accumulator register instead of materialising a zero
+          // accumulator register instead of materialising a zero.  The packed probabilities of the
+          // whole tile (NT*4 dwords) take over the registers of acc[0], whose scores are consumed by then.
           int d0 = __builtin_amdgcn_cvt_pk_fp8_f32(p[4 * q4], p[4 * q4 + 1], acc[nt][4 * q4], false);
-          pk[nt][q4] = __builtin_amdgcn_cvt_pk_fp8_f32(p[4 * q4 + 2], p[4 * q4 + 3], d0, true);
-        }
-      }
-      // ---- O^T += V^T . P^T ----
-      {
-        constexpr int NV = (BN / 64) * DTN, VPF = 2;
-        auto vfrag = [&](int i) {
-          const uint8_t* vp0 = vbuf + ((i * 2) * 64 + lane) * 16;
-          v4i lo = *reinterpret_cast<const v4i*>(vp0);
-          v4i hi = *reinterpret_cast<const v4i*>(vp0 + 64 * 16);
-          return v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-        };
-        v8i vf[NV];
-#pragma unroll
-        for (int i = 0; i < VPF; i++) vf[i] = vfrag(i);
-#pragma unroll
-        for (int i = 0; i < NV; i++) {
-          const int kk = i / DTN, dt = i % DTN;
-          if (i + VPF < NV) vf[i + VPF] = vfrag(i + VPF);
-          v8i pb;
-#pragma unroll
-          for (int e = 0; e < 4; e++) { pb[e] = pk[2 * kk][e]; pb[4 + e] = pk[2 * kk + 1][e]; }
-          if constexpr (MSUM) {
-            if (dt == 0) osum = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ones, pb, osum, 0, 0, 0, 0, 0, 0);
-          }
-          o[dt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vf[i], pb, o[dt], 0, 0, 0, 0, 0, 0);
+          acc[0][4 * nt + q4] = __builtin_amdgcn_cvt_pk_fp8_f32(p[4 * q4 + 2], p[4 * q4 + 3], d0, true);
         }
       }
     } else {
-      v8h ph[NT][2];
 #pragma unroll
       for (int nt = 0; nt < NT; nt++) {
         const float c = __builtin_fmaf(-kBiasF, sc[nt], PSHIFT - m_used);
@@ -341,33 +359,123 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
           ph[nt][r >> 3][r & 7] = (_Float16)p;
         }
       }
+    }
+    load_scales(j + 1);
+  };
+
+  // ---- O^T += V^T . P^T ----
+  auto pv = [&](int j) {
+    const uint8_t* vbuf = vslot(j);
+    if constexpr (PV == 1) {
+      constexpr int NV = (BN / 64) * DTN, VPF = 3;
+      auto vfrag = [&](int i) {
+        const uint8_t* vp0 = vbuf + ((i * 2) * 64 + lane) * 16;
+        v4i lo = *reinterpret_cast<const v4i*>(vp0);
+        v4i hi = *reinterpret_cast<const v4i*>(vp0 + 64 * 16);
+        return v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      };
+      v8i vf[NV];
 #pragma unroll
-      for (int k16 = 0; k16 < BN / 16; k16++) {
+      for (int i = 0; i < VPF; i++) vf[i] = vfrag(i);
 #pragma unroll
-        for (int dt = 0; dt < DTN; dt++) {
-          v8h va = *reinterpret_cast<const v8h*>(vbuf + ((k16 * DTN + dt) * 64 + lane) * 16);
-          o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va, ph[k16 >> 1][k16 & 1], o[dt], 0, 0, 0);
+      for (int i = 0; i < NV; i++) {
+        const int kk = i / DTN, dt = i % DTN;
+        if (i + VPF < NV) vf[i + VPF] = vfrag(i + VPF);
+        v8i pb;
+#pragma unroll
+        for (int e = 0; e < 8; e++) pb[e] = acc[0][8 * kk + e];
+        if constexpr (MSUM) {
+          if (dt == 0) osum = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ones, pb, osum, 0, 0, 0, 0, 0, 0);
         }
+        o[dt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vf[i], pb, o[dt], 0, 0, 0, 0, 0, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x100, 2 * VPF, 0);
+#pragma unroll
+      for (int i = 0; i < NV; i++) {
+        if (MSUM && i % DTN == 0) __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        if (i + VPF < NV) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+      }
+    } else {
+      constexpr int NV = (BN / 16) * DTN, VPF = 4;
+      auto vfrag = [&](int i) { return *reinterpret_cast<const v8h*>(vbuf + (i * 64 + lane) * 16); };
+      v8h vf[NV];
+#pragma unroll
+      for (int i = 0; i < VPF; i++) vf[i] = vfrag(i);
+#pragma unroll
+      for (int i = 0; i < NV; i++) {
+        const int k16 = i / DTN, dt = i % DTN;
+        if (i + VPF < NV) vf[i + VPF] = vfrag(i + VPF);
+        o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[i], ph[k16 >> 1][k16 & 1], o[dt], 0, 0, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x100, VPF, 0);
+#pragma unroll
+      for (int i = 0; i < NV; i++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        if (i + VPF < NV) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
       }
     }
   };
 
-  // ---- main loop over KV tiles ----
+  // ---- main loop: two groups of wavefronts half a tile apart ----
+  // A SIMD hosts one wavefront of each group.  In every phase one of them feeds the matrix pipe
+  // (P.V of its previous tile, then Q.K^T of its next tile) while the other runs the softmax of the
+  // tile in between on the vector ALU, and they swap at the next barrier: the two pipes of the SIMD
+  // are kept busy at the same time instead of taking turns.
+  //   phase 2j  : group 0: P.V(j-1), Q.K^T(j)      group 1: softmax(j-1)
+  //   phase 2j+1: group 0: softmax(j)              group 1: P.V(j-1), Q.K^T(j)
+  // K tile j is read in phases 2j and 2j+1, V tile j in phases 2j+2 and 2j+3; both are loaded one
+  // whole period before their first use, into the slot whose last reader finished a barrier ago.
   if (ntiles > 0) {
-    uint8_t* s0 = smem;               // tile j
-    uint8_t* s1 = smem + STAGE;       // tile j+1
-    uint8_t* s2 = smem + 2 * STAGE;   // tile j+2 (being filled)
-    load_tile(0, s0);
-    if (ntiles > 1) load_tile(1, s1);
-    for (int j = 0; j < ntiles; j++) {
-      // tile j must have landed: at most the loads of tile j+1 (issued one iteration ago) may be pending
-      if (j + 1 < ntiles) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(KPIECES + VPIECES) : "memory");
-      else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      lds_barrier();   // everyone's pieces of tile j are visible; everyone is done reading tile j-1
-      if (j + 2 < ntiles) load_tile(j + 2, s2);
-      if (j < wave_ntiles) compute(s0, j);
-      uint8_t* t = s0; s0 = s1; s1 = s2; s2 = t;
+    const int grp = (w >> GSH) & 1;
+    const int wnt = wave_ntiles;
+    auto mfma_phase = [&](int j) {
+      if (j >= 1 && j - 1 < wnt) pv(j - 1);
+      if (j < wnt) { qk(j); rowmax(j); }
+    };
+    load_k(0);
+    load_scales(0);
+#ifdef SAGE_TIMING
+    long long tacc[8] = {0, 0, 0, 0, 0, 0, 0, 0}, tlast = clock64();
+#endif
+    auto even_barrier = [&](int j) {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // my pieces of K(j) and V(j-1) have landed
+      TICK(5);
+      lds_barrier();
+      TICK(6);                                     // ... and everyone's; phase 2j-1 is over
+      if (j + 1 < ntiles) load_k(j + 1);
+      if (j < ntiles) load_v(j);
+    };
+    if (grp == 0) {
+      for (int j = 0; j <= ntiles; j++) {
+        even_barrier(j);
+        TICK(0);
+        mfma_phase(j);
+        TICK(1);
+        lds_barrier();
+        TICK(2);
+        if (j < wnt) softmax(j);
+        TICK(3);
+      }
+    } else {
+      for (int j = 0; j <= ntiles; j++) {
+        even_barrier(j);
+        TICK(0);
+        if (j >= 1 && j - 1 < wnt) softmax(j - 1);
+        TICK(3);
+        lds_barrier();
+        TICK(2);
+        mfma_phase(j);
+        TICK(1);
+      }
     }
+#ifdef SAGE_TIMING
+    if (blockIdx.x == 100 && lane == 0) {
+      for (int i = 0; i < 4; i++) g_timing[w * 8 + i] = tacc[i];
+      g_timing[w * 8 + 5] = tacc[5]; g_timing[w * 8 + 6] = tacc[6];
+      g_timing[w * 8 + 4] = ntiles;
+    }
+#endif
   }
 
   // ---- epilogue: O = O^T / l (* v_scale), LSE2 = m + log2(l) ----
@@ -468,7 +576,7 @@ AttnConfig attn_config(int D, int pv, bool packed) {
 template <int D, int NW, int BN, int PV, bool CAUSAL, bool MSUM>
 static hipError_t launch_one(const AttnArgs& a, int grid, hipStream_t st) {
   constexpr int VESZ = PV ? 1 : 2;
-  constexpr int smem = 3 * (BN * D + BN * D * VESZ);
+  constexpr int smem = 2 * (BN * D + BN * D * VESZ);   // two K slots + two V slots
   auto kern = attn_kernel<D, NW, BN, PV, CAUSAL, MSUM>;
   static bool attr_done = false;
   if (!attr_done) {
@@ -480,6 +588,9 @@ static hipError_t launch_one(const AttnArgs& a, int grid, hipStream_t st) {
   return hipGetLastError();
 }
 
+#ifdef SAGE_TIMING
+extern "C" int sage_debug_timing(long long* out) { return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_timing), sizeof(long long) * 64); }
+#endif
 hipError_t launch_attn(const AttnArgs& a, int D, int pv, bool causal, int grid, hipStream_t st) {
   if (grid == 0) return hipSuccess;
   const bool msum = pv && a.lse == nullptr;   // row sums on the matrix pipe unless LSE is wanted
