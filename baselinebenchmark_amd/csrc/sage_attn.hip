@@ -300,13 +300,15 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
         }
     }
     // ---- row maximum of this tile, in score units ----
+    // The biased scores are positive floats (or -inf where masked), so their bit patterns order like
+    // signed integers: integer max3 needs no NaN canonicalisation.
     mloc = kNegInf;
 #pragma unroll
     for (int nt = 0; nt < NT; nt++) {
-      float mx = as_f(acc[nt][0]);
+      int mx = acc[nt][0];
 #pragma unroll
-      for (int r = 1; r < 16; r++) mx = fmaxf(mx, as_f(acc[nt][r]));
-      mloc = fmaxf(mloc, __builtin_fmaf(mx, sc[nt], -kBiasF * sc[nt]));
+      for (int r = 1; r < 16; r++) mx = max(mx, acc[nt][r]);
+      mloc = fmaxf(mloc, __builtin_fmaf(as_f(mx), sc[nt], -kBiasF * sc[nt]));
     }
   };
 
@@ -341,10 +343,10 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
         }
 #pragma unroll
         for (int q4 = 0; q4 < 4; q4++) {
-          // both halves of the dword get written, so the 'old' operand is a don't-care: reuse a dead
-          // accumulator register instead of materialising a zero.  The packed probabilities of the
-          // whole tile (NT*4 dwords) take over the registers of acc[0], whose scores are consumed by then.
-          int d0 = __builtin_amdgcn_cvt_pk_fp8_f32(p[4 * q4], p[4 * q4 + 1], acc[nt][4 * q4], false);
+          // The packed probabilities of the whole tile (NT*4 dwords) take over the registers of acc[0],
+          // whose scores are consumed by then.  Both halves of each dword get written, so the 'old'
+          // operand is a don't-care: it is the destination register itself.
+          int d0 = __builtin_amdgcn_cvt_pk_fp8_f32(p[4 * q4], p[4 * q4 + 1], acc[0][4 * nt + q4], false);
           acc[0][4 * nt + q4] = __builtin_amdgcn_cvt_pk_fp8_f32(p[4 * q4 + 2], p[4 * q4 + 3], d0, true);
         }
       }
