@@ -21,20 +21,19 @@
 //     q_scale*k_scale and subtracts the running maximum.
 //   * The running maximum is only moved when it grows by more than kTau (lazy rescale); P is stored
 //     with a static 2^kPShift so that fp8's range [2^-9, 448] is used.
-//   * K/V tiles go global -> registers -> LDS, double buffered, one barrier per KV tile.
+//   * K/V tiles go global -> LDS directly (buffer_load ... lds, no registers), two slots each.
+//   * The wavefronts of a workgroup form two groups that run half a tile apart, two barriers per tile:
+//     while one group feeds the matrix pipe (P.V of its last tile, Q.K^T of its next) the other runs
+//     the softmax of the tile in between on the vector ALU.  Wavefronts w and w+4 share a SIMD and
+//     are in different groups, so each SIMD always has matrix work and vector work to overlap.
 #include "sage_launch.h"
 #include <cstdlib>
+// Bit of the wavefront index that picks the group: wavefronts w and w + 4 share a SIMD.
 #ifndef SAGE_GSH
 #define SAGE_GSH 2
 #endif
 
 namespace sage {
-#ifdef SAGE_TIMING
-__device__ long long g_timing[8 * 8];
-#define TICK(i) do { long long t_ = clock64(); tacc[i] += t_ - tlast; tlast = t_; } while (0)
-#else
-#define TICK(i)
-#endif
 
 
 constexpr float kBiasF = 12582912.0f;     // 1.5 * 2^23
@@ -314,6 +313,10 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
 
   // ---- online softmax of the tile whose scores are in acc: pure VALU work ----
   auto softmax = [&](int j) {
+    // next tile's K scales: requested first, consumed last
+    float kraw[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; nt++) kraw[nt] = ksc[min(((j + 1) * BN + 32 * nt) >> a.blkk_shift, nkblk - 1)];
     const float mall = xchg32_max(mloc);
     // lazy rescale: move the reference maximum only when it grew by more than TAU
     if (__builtin_amdgcn_ballot_w64(mall > m_used + TAU) != 0) {
@@ -362,7 +365,8 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
         }
       }
     }
-    load_scales(j + 1);
+#pragma unroll
+    for (int nt = 0; nt < NT; nt++) sc[nt] = qscale * kraw[nt];
   };
 
   // ---- O^T += V^T . P^T ----
@@ -437,47 +441,27 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
     };
     load_k(0);
     load_scales(0);
-#ifdef SAGE_TIMING
-    long long tacc[8] = {0, 0, 0, 0, 0, 0, 0, 0}, tlast = clock64();
-#endif
     auto even_barrier = [&](int j) {
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // my pieces of K(j) and V(j-1) have landed
-      TICK(5);
-      lds_barrier();
-      TICK(6);                                     // ... and everyone's; phase 2j-1 is over
+      lds_barrier();                                     // ... and everyone's; phase 2j-1 is over
       if (j + 1 < ntiles) load_k(j + 1);
       if (j < ntiles) load_v(j);
     };
     if (grp == 0) {
       for (int j = 0; j <= ntiles; j++) {
         even_barrier(j);
-        TICK(0);
         mfma_phase(j);
-        TICK(1);
         lds_barrier();
-        TICK(2);
         if (j < wnt) softmax(j);
-        TICK(3);
       }
     } else {
       for (int j = 0; j <= ntiles; j++) {
         even_barrier(j);
-        TICK(0);
         if (j >= 1 && j - 1 < wnt) softmax(j - 1);
-        TICK(3);
         lds_barrier();
-        TICK(2);
         mfma_phase(j);
-        TICK(1);
       }
     }
-#ifdef SAGE_TIMING
-    if (blockIdx.x == 100 && lane == 0) {
-      for (int i = 0; i < 4; i++) g_timing[w * 8 + i] = tacc[i];
-      g_timing[w * 8 + 5] = tacc[5]; g_timing[w * 8 + 6] = tacc[6];
-      g_timing[w * 8 + 4] = ntiles;
-    }
-#endif
   }
 
   // ---- epilogue: O = O^T / l (* v_scale), LSE2 = m + log2(l) ----
@@ -590,9 +574,6 @@ static hipError_t launch_one(const AttnArgs& a, int grid, hipStream_t st) {
   return hipGetLastError();
 }
 
-#ifdef SAGE_TIMING
-extern "C" int sage_debug_timing(long long* out) { return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_timing), sizeof(long long) * 64); }
-#endif
 hipError_t launch_attn(const AttnArgs& a, int D, int pv, bool causal, int grid, hipStream_t st) {
   if (grid == 0) return hipSuccess;
   const bool msum = pv && a.lse == nullptr;   // row sums on the matrix pipe unless LSE is wanted
