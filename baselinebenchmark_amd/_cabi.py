@@ -36,10 +36,16 @@ SIGNATURES = {
     "sage_varlen_plan": (c_int, [_P, _P, _I, _I, _I, _I, _I, _P, c_size_t, _P]),
     "sage_attn_fwd": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I,
                               _L, _L, _L, _L, _L, _L, _L, _L, _L, _I, _I, _I, _I, _I, _P, _P, _P, _I, _L, _L, _L, _P]),
+    "sage_attn_fwd_masked": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I,
+                                     _L, _L, _L, _L, _L, _L, _L, _L, _L, _I, _I, _I, _I, _P, _I, _L, _L, _L, _L, _P]),
     "sage_sageattn_workspace_bytes": (c_size_t, [_I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I]),
     "sage_sageattn": (c_int, [_P, _P, _P, _P, _P, _P, c_size_t, _I, _I, _I, _I, _I, _I,
                               _L, _L, _L, _L, _L, _L, _L, _L, _L, _L, _L, _L,
                               _I, _I, _I, c_double, _I, _I, _I, _P, _P, _I, _I, _P]),
+    "sage_sageattn_masked": (c_int, [_P, _P, _P, _P, _P, _P, c_size_t, _I, _I, _I, _I, _I, _I,
+                                     _L, _L, _L, _L, _L, _L, _L, _L, _L, _L, _L, _L,
+                                     _I, _I, _I, c_double, _I, _I, _I, _P, _P, _I, _I,
+                                     _P, _I, _L, _L, _L, _L, _P]),
 }
 
 _lib = None

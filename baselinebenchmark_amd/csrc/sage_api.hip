@@ -56,10 +56,20 @@ const char* sage_backend_name(void) { return "mi355x_hip_int8_qk_fp8_fp16_pv"; }
 
 const char* sage_last_error(void) { return g_err; }
 
-int sage_quant_int8(const void* x, int8_t* out, float* scale, const void* km, int B, int H, int L, int D, int64_t x_sb,
-                    int64_t x_sh, int64_t x_sn, int64_t o_sb, int64_t o_sh, int64_t o_sn, int64_t km_sb, int64_t km_sh,
-                    int blk, float mult, int dtype, const int32_t* cu_seqlens, const int32_t* cu_blocks,
-                    int64_t scale_sh, sage_stream_t stream) {
+}  // extern "C"
+
+namespace {
+struct RowDot {   // optional side output of the quantiser (see QuantArgs)
+  const void* vec = nullptr;
+  float* out = nullptr;
+  int64_t sb = 0, sh = 0;
+  int group = 1, total = 0;
+};
+
+int quant_impl(const void* x, int8_t* out, float* scale, const void* km, int B, int H, int L, int D, int64_t x_sb,
+               int64_t x_sh, int64_t x_sn, int64_t o_sb, int64_t o_sh, int64_t o_sn, int64_t km_sb, int64_t km_sh, int blk,
+               float mult, int dtype, const int32_t* cu_seqlens, const int32_t* cu_blocks, int64_t scale_sh,
+               const RowDot& dot, sage_stream_t stream) {
   if (int rc = check_common(B, H, L, D, dtype)) return rc;
   if (!valid_blk_quant(blk)) return fail(SAGE_ENOTIMPL, "quantisation block %d is not supported (16, 32, 64, 128)", blk);
   if (B == 0 || H == 0 || L == 0) return SAGE_OK;
@@ -69,14 +79,28 @@ int sage_quant_int8(const void* x, int8_t* out, float* scale, const void* km, in
   if (int rc = check_stride16("out", o_sb, o_sh, o_sn, 1, out)) return rc;
   if (km && int(check_stride16("km", km_sb, km_sh, 0, 2, km))) return SAGE_EINVAL;
   QuantArgs a;
+  memset(&a, 0, sizeof(a));
   a.x = (const u16*)x; a.out = out; a.scale = scale; a.km = (const u16*)km;
   a.B = B; a.H = H; a.L = L; a.D = D;
   a.x_sb = x_sb; a.x_sh = x_sh; a.x_sn = x_sn; a.o_sb = o_sb; a.o_sh = o_sh; a.o_sn = o_sn;
   a.km_sb = km_sb; a.km_sh = km_sh; a.blk = blk; a.mult = mult;
   a.cu_seqlens = cu_seqlens; a.cu_blocks = cu_blocks; a.scale_sh = scale_sh;
+  a.dotv = (const u16*)dot.vec; a.dot_out = dot.out; a.dv_sb = dot.sb; a.dv_sh = dot.sh; a.dv_group = dot.group;
+  a.dot_total = dot.total;
   hipError_t e = launch_quant_int8(a, dtype, (L + blk - 1) / blk, (hipStream_t)stream);
   if (e != hipSuccess) return hip_fail(e, "sage_quant_int8");
   return SAGE_OK;
+}
+}  // namespace
+
+extern "C" {
+
+int sage_quant_int8(const void* x, int8_t* out, float* scale, const void* km, int B, int H, int L, int D, int64_t x_sb,
+                    int64_t x_sh, int64_t x_sn, int64_t o_sb, int64_t o_sh, int64_t o_sn, int64_t km_sb, int64_t km_sh,
+                    int blk, float mult, int dtype, const int32_t* cu_seqlens, const int32_t* cu_blocks,
+                    int64_t scale_sh, sage_stream_t stream) {
+  return quant_impl(x, out, scale, km, B, H, L, D, x_sb, x_sh, x_sn, o_sb, o_sh, o_sn, km_sb, km_sh, blk, mult, dtype,
+                    cu_seqlens, cu_blocks, scale_sh, RowDot(), stream);
 }
 
 size_t sage_k_mean_workspace_bytes(int B, int H, int L, int D) {
@@ -158,12 +182,22 @@ int sage_varlen_plan(const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k, i
   return SAGE_OK;
 }
 
-int sage_attn_fwd(const int8_t* q, const int8_t* k, const void* v_panels, const float* q_scale, const float* k_scale,
-                  const float* v_scale, void* out, float* lse, int B, int Hq, int Hkv, int Sq, int Skv, int D, int64_t q_sb,
-                  int64_t q_sh, int64_t q_sn, int64_t k_sb, int64_t k_sh, int64_t k_sn, int64_t o_sb, int64_t o_sh,
-                  int64_t o_sn, int blkq, int blkk, int is_causal, int pv_mode, int out_dtype, const int32_t* cu_seqlens_q,
-                  const int32_t* cu_seqlens_k, const int32_t* plan, int total_q, int64_t q_scale_sh, int64_t k_scale_sh,
-                  int64_t panel_sh, sage_stream_t stream) {
+}  // extern "C"
+
+namespace {
+struct MaskArg {
+  const void* ptr = nullptr;
+  int kind = 0;
+  int64_t sb = 0, sh = 0, sm = 0, sn = 0;
+  float mult = 1.0f;   // additive masks are multiplied by this (1 for base-2 units, log2(e) for natural units)
+};
+
+int attn_impl(const int8_t* q, const int8_t* k, const void* v_panels, const float* q_scale, const float* k_scale,
+              const float* v_scale, void* out, float* lse, int B, int Hq, int Hkv, int Sq, int Skv, int D, int64_t q_sb,
+              int64_t q_sh, int64_t q_sn, int64_t k_sb, int64_t k_sh, int64_t k_sn, int64_t o_sb, int64_t o_sh,
+              int64_t o_sn, int blkq, int blkk, int is_causal, int pv_mode, int out_dtype, const int32_t* cu_seqlens_q,
+              const int32_t* cu_seqlens_k, const int32_t* plan, int total_q, int64_t q_scale_sh, int64_t k_scale_sh,
+              int64_t panel_sh, const MaskArg& mask, const float* lse_offset, sage_stream_t stream) {
   if (int rc = check_common(B, Hq, Sq, D, out_dtype)) return rc;
   if (Hkv <= 0 || Hq % Hkv) return fail(SAGE_EINVAL, "query heads (%d) must be divisible by KV heads (%d)", Hq, Hkv);
   if (Skv < 0) return fail(SAGE_EINVAL, "negative kv length");
@@ -178,6 +212,12 @@ int sage_attn_fwd(const int8_t* q, const int8_t* k, const void* v_panels, const 
   if ((o_sb % 4) || (o_sh % 4) || (o_sn % 4) || reinterpret_cast<uintptr_t>(out) % 8)
     return fail(SAGE_EINVAL, "out: base pointer and strides must be 8-byte aligned");
   const bool packed = cu_seqlens_q != nullptr;
+  if (mask.ptr) {
+    if (mask.kind != SAGE_MASK_BOOL && mask.kind != SAGE_MASK_ADDITIVE) return fail(SAGE_EINVAL, "mask kind %d unknown", mask.kind);
+    if (packed) return fail(SAGE_ENOTIMPL, "an explicit mask is not supported for packed batches");
+    if (is_causal) return fail(SAGE_ENOTIMPL, "an explicit mask cannot be combined with is_causal");
+    if (mask.kind == SAGE_MASK_ADDITIVE && reinterpret_cast<uintptr_t>(mask.ptr) % 4) return fail(SAGE_EINVAL, "additive mask must be 4-byte aligned");
+  }
   if (packed && (!cu_seqlens_k || !plan)) return fail(SAGE_EINVAL, "packed mode needs cu_seqlens_k and plan");
   if (packed && B > 32767) return fail(SAGE_EINVAL, "too many sequences");
   AttnConfig cfg = attn_config(D, pv_mode, packed);
@@ -191,7 +231,8 @@ int sage_attn_fwd(const int8_t* q, const int8_t* k, const void* v_panels, const 
   a.o_sb = o_sb; a.o_sh = o_sh; a.o_sn = o_sn;
   a.blkq = blkq; a.blkk = blkk; a.blkq_shift = ilog2(blkq); a.blkk_shift = ilog2(blkk); a.out_bf16 = out_dtype == SAGE_DT_BF16;
   a.nqt = (Sq + BM - 1) / BM;
-  { const char* e = getenv("SAGE_PP_SPLIT"); a.pp_split = e ? atoi(e) : 0; }
+  a.mask = mask.ptr; a.mask_kind = mask.kind; a.m_sb = mask.sb; a.m_sh = mask.sh; a.m_sm = mask.sm; a.m_sn = mask.sn;
+  a.mask_mult = mask.mult; a.lse_offset = lse_offset;
   int64_t grid;
   if (packed) {
     SagePlanLayout L = plan_layout(B, total_q);
@@ -208,11 +249,36 @@ int sage_attn_fwd(const int8_t* q, const int8_t* k, const void* v_panels, const 
   if (e != hipSuccess) return hip_fail(e, "sage_attn_fwd");
   return SAGE_OK;
 }
+}  // namespace
+
+extern "C" {
+
+int sage_attn_fwd(const int8_t* q, const int8_t* k, const void* v_panels, const float* q_scale, const float* k_scale,
+                  const float* v_scale, void* out, float* lse, int B, int Hq, int Hkv, int Sq, int Skv, int D, int64_t q_sb,
+                  int64_t q_sh, int64_t q_sn, int64_t k_sb, int64_t k_sh, int64_t k_sn, int64_t o_sb, int64_t o_sh,
+                  int64_t o_sn, int blkq, int blkk, int is_causal, int pv_mode, int out_dtype, const int32_t* cu_seqlens_q,
+                  const int32_t* cu_seqlens_k, const int32_t* plan, int total_q, int64_t q_scale_sh, int64_t k_scale_sh,
+                  int64_t panel_sh, sage_stream_t stream) {
+  return attn_impl(q, k, v_panels, q_scale, k_scale, v_scale, out, lse, B, Hq, Hkv, Sq, Skv, D, q_sb, q_sh, q_sn, k_sb, k_sh, k_sn, o_sb, o_sh, o_sn, blkq, blkk, is_causal, pv_mode, out_dtype, cu_seqlens_q, cu_seqlens_k, plan, total_q, q_scale_sh, k_scale_sh, panel_sh, MaskArg(), nullptr, stream);
+}
+
+int sage_attn_fwd_masked(const int8_t* q, const int8_t* k, const void* v_panels, const float* q_scale, const float* k_scale,
+                         const float* v_scale, void* out, float* lse, int B, int Hq, int Hkv, int Sq, int Skv, int D,
+                         int64_t q_sb, int64_t q_sh, int64_t q_sn, int64_t k_sb, int64_t k_sh, int64_t k_sn, int64_t o_sb,
+                         int64_t o_sh, int64_t o_sn, int blkq, int blkk, int pv_mode, int out_dtype, const void* attn_mask,
+                         int mask_kind, int64_t m_sb, int64_t m_sh, int64_t m_sm, int64_t m_sn, sage_stream_t stream) {
+  if (!attn_mask) return fail(SAGE_EINVAL, "null mask");
+  MaskArg m;
+  m.ptr = attn_mask; m.kind = mask_kind; m.sb = m_sb; m.sh = m_sh; m.sm = m_sm; m.sn = m_sn;
+  return attn_impl(q, k, v_panels, q_scale, k_scale, v_scale, out, lse, B, Hq, Hkv, Sq, Skv, D, q_sb, q_sh, q_sn, k_sb, k_sh,
+                   k_sn, o_sb, o_sh, o_sn, blkq, blkk, 0, pv_mode, out_dtype, nullptr, nullptr, nullptr, 0, 0, 0, 0, m, nullptr,
+                   stream);
+}
 
 // ---- one-call pipeline --------------------------------------------------------------------
 namespace {
 struct E2EWorkspace {
-  size_t q_i8, k_i8, q_scale, k_scale, km, v_scale, panels, stat, plan, total;
+  size_t q_i8, k_i8, q_scale, k_scale, km, v_scale, panels, stat, plan, lse_off, total;
   int64_t qs_sh, ks_sh, panel_sh;
 };
 E2EWorkspace e2e_layout(int B, int Hq, int Hkv, int Sq, int Skv, int D, int blkq, int blkk, int pv, int total_q, int total_k,
@@ -240,6 +306,7 @@ E2EWorkspace e2e_layout(int B, int Hq, int Hkv, int Sq, int Skv, int D, int blkq
   size_t stat2 = sage_prep_v_workspace_bytes(B, Hkv, Skv, D, pv);
   w.stat = off; off += align_up(stat > stat2 ? stat : stat2);
   w.plan = off; off += varlen ? align_up(sage_varlen_plan_ints(B, total_q) * 4) : 0;
+  w.lse_off = off; off += align_up((varlen ? (size_t)Hq * total_q : (size_t)B * Hq * Sq) * 4);
   w.total = off;
   return w;
 }
@@ -256,6 +323,18 @@ int sage_sageattn(const void* q, const void* k, const void* v, void* out, float*
                   int64_t k_sh, int64_t k_sn, int64_t v_sb, int64_t v_sh, int64_t v_sn, int64_t o_sb, int64_t o_sh,
                   int64_t o_sn, int dtype, int blkq, int blkk, double sm_scale, int is_causal, int smooth_k, int pv_mode,
                   const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k, int total_q, int total_k, sage_stream_t stream) {
+  return sage_sageattn_masked(q, k, v, out, lse, workspace, workspace_bytes, B, Hq, Hkv, Sq, Skv, D, q_sb, q_sh, q_sn, k_sb,
+                              k_sh, k_sn, v_sb, v_sh, v_sn, o_sb, o_sh, o_sn, dtype, blkq, blkk, sm_scale, is_causal, smooth_k,
+                              pv_mode, cu_seqlens_q, cu_seqlens_k, total_q, total_k, nullptr, 0, 0, 0, 0, 0, stream);
+}
+
+int sage_sageattn_masked(const void* q, const void* k, const void* v, void* out, float* lse, void* workspace,
+                         size_t workspace_bytes, int B, int Hq, int Hkv, int Sq, int Skv, int D, int64_t q_sb, int64_t q_sh,
+                         int64_t q_sn, int64_t k_sb, int64_t k_sh, int64_t k_sn, int64_t v_sb, int64_t v_sh, int64_t v_sn,
+                         int64_t o_sb, int64_t o_sh, int64_t o_sn, int dtype, int blkq, int blkk, double sm_scale,
+                         int is_causal, int smooth_k, int pv_mode, const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+                         int total_q, int total_k, const void* attn_mask, int mask_kind, int64_t m_sb, int64_t m_sh,
+                         int64_t m_sm, int64_t m_sn, sage_stream_t stream) {
   if (int rc = check_common(B, Hq, Sq, D, dtype)) return rc;
   if (Hkv <= 0 || Hq % Hkv) return fail(SAGE_EINVAL, "query heads (%d) must be divisible by KV heads (%d)", Hq, Hkv);
   if (!valid_blk_attn(blkq) || !valid_blk_attn(blkk))
@@ -297,15 +376,30 @@ int sage_sageattn(const void* q, const void* k, const void* v, void* out, float*
   rc = sage_quant_int8(k, k_i8, k_scale, smooth_k ? km : nullptr, B, Hkv, Skv, D, k_sb, k_sh, k_sn, k_sb, k_sh, k_sn,
                        (int64_t)Hkv * D, D, blkk, 1.0f, dtype, cu_seqlens_k, cu_kblk, w.ks_sh, stream);
   if (rc) return rc;
-  rc = sage_quant_int8(q, q_i8, q_scale, nullptr, B, Hq, Sq, D, q_sb, q_sh, q_sn, q_sb, q_sh, q_sn, 0, 0, blkq,
-                       (float)((sm_scale > 0 ? sm_scale : 1.0 / sqrt((double)D)) * 1.44269504), dtype, cu_seqlens_q, cu_qblk, w.qs_sh, stream);
+  // With K smoothing every logit of a query row loses q . k_mean; the softmax does not notice but the
+  // log-sum-exp does, so when LSE is requested the Q quantiser also emits that dot product (in the
+  // base-2 units of the scaled Q) and the attention kernel adds it back.
+  RowDot dot;
+  float* lse_off = nullptr;
+  if (lse && smooth_k) {
+    lse_off = (float*)(ws + w.lse_off);
+    dot.vec = km; dot.out = lse_off; dot.sb = (int64_t)Hkv * D; dot.sh = D; dot.group = Hq / Hkv; dot.total = total_q;
+  }
+  rc = quant_impl(q, q_i8, q_scale, nullptr, B, Hq, Sq, D, q_sb, q_sh, q_sn, q_sb, q_sh, q_sn, 0, 0, blkq,
+                  (float)((sm_scale > 0 ? sm_scale : 1.0 / sqrt((double)D)) * 1.44269504), dtype, cu_seqlens_q, cu_qblk, w.qs_sh,
+                  dot, stream);
   if (rc) return rc;
   rc = sage_prep_v(v, panels, v_scale, stat, stat_bytes, B, Hkv, Skv, D, v_sb, v_sh, v_sn, dtype, pv_mode, cu_seqlens_k,
                    cu_panel, w.panel_sh, stream);
   if (rc) return rc;
-  return sage_attn_fwd(q_i8, k_i8, panels, q_scale, k_scale, pv_mode == SAGE_PV_FP8 ? v_scale : nullptr, out, lse, B, Hq, Hkv,
-                       Sq, Skv, D, q_sb, q_sh, q_sn, k_sb, k_sh, k_sn, o_sb, o_sh, o_sn, blkq, blkk, is_causal, pv_mode, dtype,
-                       cu_seqlens_q, cu_seqlens_k, plan, total_q, w.qs_sh, w.ks_sh, w.panel_sh, stream);
+  MaskArg m;
+  if (attn_mask) {
+    // sageattn's additive mask is in natural-log units on top of sm_scale * q.k (test_sage_attention_mate.py:171-176)
+    m.ptr = attn_mask; m.kind = mask_kind; m.sb = m_sb; m.sh = m_sh; m.sm = m_sm; m.sn = m_sn; m.mult = 1.44269504f;
+  }
+  return attn_impl(q_i8, k_i8, panels, q_scale, k_scale, pv_mode == SAGE_PV_FP8 ? v_scale : nullptr, out, lse, B, Hq, Hkv, Sq,
+                   Skv, D, q_sb, q_sh, q_sn, k_sb, k_sh, k_sn, o_sb, o_sh, o_sn, blkq, blkk, is_causal, pv_mode, dtype,
+                   cu_seqlens_q, cu_seqlens_k, plan, total_q, w.qs_sh, w.ks_sh, w.panel_sh, m, lse_off, stream);
 }
 
 }  // extern "C"

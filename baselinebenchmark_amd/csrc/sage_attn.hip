@@ -1,496 +1,7 @@
-// Fused SageAttention forward kernel for gfx950 (MI355X).
-//
-// Replaces _attention_kernel of backends/_hygon/ops/sageattention/sageattention_triton.py:45-129
-// (INT8 Q.K^T, fp32 base-2 online softmax, P.V with fp32 accumulation, O/l epilogue, LSE2) and adds
-// causal block skipping, tail masking, FP8 P.V and packed variable-length batches.
-//
-// Mapping to the hardware
-//   * A workgroup of NW wavefronts owns a q-tile of BM = 32*NW rows of one (batch, q-head); each
-//     wavefront owns 32 query rows for the whole KV loop.
-//   * Everything is computed TRANSPOSED so that a query row lives in one lane column:
-//       S^T[n, m] = K[n, :] . Q[m, :]      v_mfma_i32_32x32x32_i8      A = K tile (LDS), B = Q (regs)
-//       O^T[d, m] = V^T[d, n] . P^T[n, m]   v_mfma_f32_32x32x64_f8f6f4  A = V panel (LDS), B = P (regs)
-//                                       or  v_mfma_f32_32x32x16_f16
-//     In the 32x32 accumulator layout lane (m = lane%32, h = lane/32) holds column m, rows
-//     8*(r/4) + 4*h + r%4.  So row max / row sum of query row m are in-lane reductions plus ONE
-//     exchange with lane m+32 (v_permlane32_swap), the probabilities are already laid out as the
-//     B operand of the second MFMA (V panels are pre-permuted to match, see sage_common.h), and the
-//     running rescale / final 1/l multiply the lane's own accumulators.
-//   * The INT32 accumulators start from the bit pattern of 1.5*2^23, so reading them as floats gives
-//     12582912 + dot exactly: the int->float conversion is folded into the one FMA that applies
-//     q_scale*k_scale and subtracts the running maximum.
-//   * The running maximum is only moved when it grows by more than kTau (lazy rescale); P is stored
-//     with a static 2^kPShift so that fp8's range [2^-9, 448] is used.
-//   * K/V tiles go global -> LDS directly (buffer_load ... lds, no registers), two slots each.
-//   * The wavefronts of a workgroup form two groups that run half a tile apart, two barriers per tile:
-//     while one group feeds the matrix pipe (P.V of its last tile, Q.K^T of its next) the other runs
-//     the softmax of the tile in between on the vector ALU.  Wavefronts w and w+4 share a SIMD and
-//     are in different groups, so each SIMD always has matrix work and vector work to overlap.
-#include "sage_launch.h"
-#include <cstdlib>
-// Bit of the wavefront index that picks the group: wavefronts w and w + 4 share a SIMD.
-#ifndef SAGE_GSH
-#define SAGE_GSH 2
-#endif
+// Launchers of the fused attention kernel (variants without an explicit mask) and the packed-batch plan.
+#include "sage_attn_kernel.h"
 
 namespace sage {
-
-
-constexpr float kBiasF = 12582912.0f;     // 1.5 * 2^23
-constexpr int kBiasBits = 0x4B400000;     // its bit pattern; int accumulators start here
-constexpr float kNegInf = -__builtin_inff();
-constexpr float kMInit = -1.0e30f;
-
-template <int PV> struct PCfg;
-template <> struct PCfg<1> { static constexpr float tau = 3.0f, pshift = 5.0f; };   // fp8: p*32 <= 256 < 448
-template <> struct PCfg<0> { static constexpr float tau = 8.0f, pshift = 0.0f; };   // fp16: p <= 256
-
-// NOTE: __builtin_bit_cast applied directly to an element of an ext_vector_type value reads element
-// 0 whatever the index (clang miscompiles the element lvalue), so vector elements are always passed
-// BY VALUE through these two helpers.
-__device__ inline float as_f(int v) { return __builtin_bit_cast(float, v); }
-__device__ inline int as_i(float v) { return __builtin_bit_cast(int, v); }
-
-// Exchange between lane l and lane l^32 (the two lanes that share a query row).
-// v_permlane32_swap swaps the upper half of its first operand with the lower half of its second, so
-// with both operands holding x every lane ends up with {x[l%32], x[l%32 + 32]}.
-__device__ inline void xchg32(float x, float& lo, float& hi) {
-  auto r = __builtin_amdgcn_permlane32_swap(as_i(x), as_i(x), false, false);
-  int r0 = r[0], r1 = r[1];
-  lo = as_f(r0);
-  hi = as_f(r1);
-}
-__device__ inline float xchg32_max(float x) {
-  float lo, hi;
-  xchg32(x, lo, hi);
-  return fmaxf(lo, hi);
-}
-__device__ inline float xchg32_sum(float x) {
-  float lo, hi;
-  xchg32(x, lo, hi);
-  return lo + hi;
-}
-
-// Workgroup barrier that only orders LDS traffic: waits for this wavefront's outstanding LDS
-// operations, then s_barrier (global-memory traffic issued ahead stays in flight).
-__device__ inline void lds_barrier() {
-  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-}
-
-// 16-byte-chunk swizzle of a K row in LDS: consecutive rows read the same logical chunk from
-// different bank groups (64 banks x 4 bytes = 256 bytes per bank row).
-template <int D>
-__device__ inline int kswz(int n) {
-  constexpr int CPR = D / 16, RPB = 256 / D;
-  return (n / RPB) % CPR;
-}
-
-template <int D, int NW, int BN, int PV, bool CAUSAL, bool MSUM>
-__global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
-  constexpr int GSH = SAGE_GSH;   // which bit of the wavefront index picks the group
-  constexpr int BM = NW * 32;
-  constexpr int NTHR = NW * 64;
-  constexpr int KS = D / 32;   // contraction steps of S^T
-  constexpr int NT = BN / 32;  // 32-row tiles of S^T
-  constexpr int DTN = D / 32;  // 32-row tiles of O^T
-  constexpr int VESZ = PV ? 1 : 2;
-  constexpr int KBYTES = BN * D, VBYTES = BN * D * VESZ, STAGE = KBYTES + VBYTES;
-  constexpr int KCHUNKS = KBYTES / 16, VCHUNKS = VBYTES / 16;
-  constexpr int PANEL_BYTES = kPanelRows * D * VESZ;
-  constexpr int CPR = D / 16;
-  constexpr float TAU = PCfg<PV>::tau, PSHIFT = PCfg<PV>::pshift;
-
-  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);  // wavefront index: uniform, keep it scalar
-  const int m = lane & 31, h = lane >> 5;
-
-  // ---- which tile am I: heaviest q-tiles first; q-heads sharing a KV head on one XCD ----
-  const bool packed = a.cu_q != nullptr;
-  const int G = a.Hq / a.Hkv;
-  int rank, s, NG;
-  if (packed) { rank = blockIdx.x / a.Hq; s = blockIdx.x % a.Hq; NG = a.Hkv; }
-  else { int U = a.B * a.Hq; rank = blockIdx.x / U; s = blockIdx.x % U; NG = a.B * a.Hkv; }
-  int gi, g;
-  if ((NG & 7) == 0) { int x = s & 7, y = s >> 3; gi = x + 8 * (y / G); g = y % G; }
-  else { gi = s / G; g = s % G; }
-  int b, kvh, qt, Lq, Lk;
-  int64_t qoff, koff, ooff, lseoff;
-  const float *qsp, *ksp;
-  const uint8_t* vbase;
-  int nkblk;
-  if (packed) {
-    if (rank >= a.ntiles[0]) return;
-    int t = a.tiles[rank];
-    b = t >> 16; qt = t & 0xffff; kvh = gi;
-    int q0 = a.cu_q[b], k0 = a.cu_k[b];
-    Lq = a.cu_q[b + 1] - q0; Lk = a.cu_k[b + 1] - k0;
-    int hq = kvh * G + g;
-    qoff = (int64_t)q0 * a.q_sn + (int64_t)hq * a.q_sh;
-    ooff = (int64_t)q0 * a.o_sn + (int64_t)hq * a.o_sh;
-    koff = (int64_t)k0 * a.k_sn + (int64_t)kvh * a.k_sh;
-    lseoff = (int64_t)hq * a.total_q + q0;
-    qsp = a.qs + (int64_t)hq * a.qs_sh + a.cu_qblk[b];
-    ksp = a.ks + (int64_t)kvh * a.ks_sh + a.cu_kblk[b];
-    vbase = a.vp + ((int64_t)kvh * a.panel_sh + a.cu_panel[b]) * PANEL_BYTES;
-  } else {
-    b = gi / a.Hkv; kvh = gi % a.Hkv;
-    qt = CAUSAL ? a.nqt - 1 - rank : rank;
-    Lq = a.Sq; Lk = a.Skv;
-    int hq = kvh * G + g;
-    qoff = (int64_t)b * a.q_sb + (int64_t)hq * a.q_sh;
-    ooff = (int64_t)b * a.o_sb + (int64_t)hq * a.o_sh;
-    koff = (int64_t)b * a.k_sb + (int64_t)kvh * a.k_sh;
-    lseoff = ((int64_t)b * a.Hq + hq) * a.Sq;
-    qsp = a.qs + ((int64_t)b * a.Hq + hq) * ((Lq + a.blkq - 1) / a.blkq);
-    ksp = a.ks + ((int64_t)b * a.Hkv + kvh) * ((Lk + a.blkk - 1) / a.blkk);
-    vbase = a.vp + ((int64_t)b * a.Hkv + kvh) * ((Lk + kPanelRows - 1) / kPanelRows) * PANEL_BYTES;
-  }
-  nkblk = (Lk + a.blkk - 1) / a.blkk;
-  // The K scales are read through the scalar cache (constant address space): a vector load would sit
-  // in the same in-order counter as the tile loads in flight and make every tile wait for them.
-  const __attribute__((address_space(4))) float* ksc = (const __attribute__((address_space(4))) float*)ksp;
-
-  const int row0 = qt * BM + w * 32;   // first query row of this wavefront
-  const int my_row = row0 + m;
-  const int kv_end = CAUSAL ? min(Lk, qt * BM + BM) : Lk;
-  const int ntiles = (kv_end + BN - 1) / BN;
-  const int wave_end = (row0 < Lq) ? (CAUSAL ? min(Lk, row0 + 32) : Lk) : 0;
-  const int wave_ntiles = (wave_end + BN - 1) / BN;
-
-  // ---- Q operand: lane (m, h) holds bytes 32*ks + 16*h .. +15 of its row for every ks ----
-  v4i qreg[KS];
-  {
-    const int8_t* qp = a.q + qoff + (int64_t)min(my_row, Lq - 1) * a.q_sn + 16 * h;
-#pragma unroll
-    for (int ks = 0; ks < KS; ks++) qreg[ks] = *reinterpret_cast<const v4i*>(qp + 32 * ks);
-  }
-  const float qscale = qsp[min(row0, Lq - 1) >> a.blkq_shift];
-
-  v16i bias;
-#pragma unroll
-  for (int i = 0; i < 16; i++) bias[i] = kBiasBits;
-  asm volatile("" : "+v"(bias));  // keep it in registers: it is the C operand of every first MFMA
-
-  v16f o[DTN];
-#pragma unroll
-  for (int dt = 0; dt < DTN; dt++)
-#pragma unroll
-    for (int i = 0; i < 16; i++) o[dt][i] = 0.f;
-  float m_used = kMInit, lsum = 0.f;
-  // MSUM (FP8 mode when no LSE is requested): the row sums come out of the matrix pipe too.  A V^T operand of all ones (fp8 1.0 = 0x38)
-  // makes every row of one extra 32x32 output tile equal to sum_n P[n][m], i.e. the softmax
-  // denominator of query row m -- of the very fp8 values that multiply V.  That removes one VALU add
-  // per score (the VALU, not the MFMA pipe, is the busier unit of this kernel).  The sum of rounded
-  // values is the right denominator for O but costs LSE accuracy on rows with few keys, so kernels
-  // that return LSE keep the fp32 VALU sum.
-  v16f osum;
-#pragma unroll
-  for (int i = 0; i < 16; i++) osum[i] = 0.f;
-  v8i ones;
-#pragma unroll
-  for (int i = 0; i < 8; i++) ones[i] = 0x38383838;
-  asm volatile("" : "+v"(ones));
-
-  // ---- tile loads: global memory -> LDS directly (no registers), 1 KB per wavefront instruction ----
-  // Lane l of a wavefront writes LDS bytes [16*l, 16*l+16) of the 1 KB piece, so the K swizzle is
-  // applied on the global side: the lane fetches the 16-byte chunk that belongs in its slot.
-  // K tiles and V tiles each alternate between two LDS slots.
-  constexpr int KPIECES = KBYTES / 1024 / NW, VPIECES = VBYTES / 1024 / NW;
-  static_assert(KPIECES * 1024 * NW == KBYTES && VPIECES * 1024 * NW == VBYTES, "tile must split into 1 KB pieces per wavefront");
-  // The buffer form of the LDS load is used on purpose: the compiler treats the global form as a flat
-  // access that may touch LDS and then drains every counter at each LDS read while one is in flight.
-  const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc((void*)(a.k + koff), 0, 0x7fffffff, 0x00020000);
-  const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc((void*)vbase, 0, 0x7fffffff, 0x00020000);
-  auto dma16 = [&](__amdgpu_buffer_rsrc_t rsrc, int lane_offset, int uniform_offset, uint8_t* dst_uniform) {
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)dst_uniform, 16, lane_offset, uniform_offset, 0, 0);
-  };
-  auto kslot = [&](int j) { return smem + (j & 1) * KBYTES; };
-  auto vslot = [&](int j) { return smem + 2 * KBYTES + (j & 1) * VBYTES; };
-  // Per-lane byte offsets of this wavefront's pieces inside a tile are loop invariant; the tile index
-  // only adds a uniform term.  Rows past the end of the sequence (last tile only) are clamped.
-  int koffv[KPIECES], voffv[VPIECES];
-#pragma unroll
-  for (int i = 0; i < KPIECES; i++) {
-    const int sl = (i * NW + w) * 64 + lane, n = sl / CPR, cc = (sl % CPR) ^ kswz<D>(n);
-    koffv[i] = n * (int)a.k_sn + 16 * cc;
-  }
-#pragma unroll
-  for (int i = 0; i < VPIECES; i++) voffv[i] = (i * NW + w) * 1024 + lane * 16;
-  const int ktile_bytes = BN * (int)a.k_sn;
-  auto load_k = [&](int j) {
-    uint8_t* dst = kslot(j);
-    if (j * BN + BN <= Lk) {
-#pragma unroll
-      for (int i = 0; i < KPIECES; i++) dma16(krsrc, koffv[i], j * ktile_bytes, dst + (i * NW + w) * 1024);
-    } else {
-#pragma unroll
-      for (int i = 0; i < KPIECES; i++) {
-        const int sl = (i * NW + w) * 64 + lane, n = sl / CPR, cc = (sl % CPR) ^ kswz<D>(n);
-        dma16(krsrc, min(j * BN + n, Lk - 1) * (int)a.k_sn + 16 * cc, 0, dst + (i * NW + w) * 1024);
-      }
-    }
-  };
-  auto load_v = [&](int j) {
-    uint8_t* dst = vslot(j);
-#pragma unroll
-    for (int i = 0; i < VPIECES; i++) dma16(vrsrc, voffv[i], j * VBYTES, dst + (i * NW + w) * 1024);
-  };
-
-  // State that crosses phases: the raw scores of the tile in flight, its row maximum and scales, and
-  // the probabilities packed as the B operand of the second MFMA.
-  v16i acc[NT];
-  float sc[NT];
-  float mloc = kNegInf;
-  v8h ph[NT][2];      // fp16 mode
-
-  // ---- S^T = K . Q^T (int8 -> int32 on the biased accumulators), then mask and row maximum ----
-  auto qk = [&](int j) {
-    const uint8_t* kbuf = kslot(j);
-    // K fragments run KPF MFMAs ahead of their use so that no MFMA waits for the LDS read issued
-    // just before it; the k-step is the outer index so that consecutive MFMAs hit different accumulators.
-    {
-      constexpr int NF = NT * KS, KPF = 4;
-      auto kfrag = [&](int i) {
-        const int nt = i % NT, ks = i / NT, n = 32 * nt + m;
-        return *reinterpret_cast<const v4i*>(kbuf + n * D + 16 * ((2 * ks + h) ^ kswz<D>(n)));
-      };
-      v4i kf[NF];
-#pragma unroll
-      for (int i = 0; i < KPF; i++) kf[i] = kfrag(i);
-#pragma unroll
-      for (int i = 0; i < NF; i++) {
-        if (i + KPF < NF) kf[i + KPF] = kfrag(i + KPF);
-        const int nt = i % NT, ks = i / NT;
-        acc[nt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf[i], qreg[ks], ks == 0 ? bias : acc[nt], 0, 0, 0);
-      }
-      __builtin_amdgcn_sched_group_barrier(0x100, KPF, 0);
-#pragma unroll
-      for (int i = 0; i < NF - KPF; i++) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      }
-      __builtin_amdgcn_sched_group_barrier(0x008, KPF, 0);
-    }
-  };
-  // q_scale * k_scale of the 32-key groups of tile j.  Fetched during the vector-ALU phase: a scalar
-  // load in flight while K/V fragments are being read would force every LDS wait to drain the queue.
-  auto load_scales = [&](int j) {
-#pragma unroll
-    for (int nt = 0; nt < NT; nt++) sc[nt] = qscale * ksc[min((j * BN + 32 * nt) >> a.blkk_shift, nkblk - 1)];
-  };
-
-  auto rowmax = [&](int j) {
-    const int n0 = j * BN;
-    // ---- masking: only tiles that cross the diagonal or the end of the sequence ----
-    const bool need_mask = (CAUSAL && (n0 + BN - 1 > row0)) || (n0 + BN > Lk);
-    if (need_mask) {
-      const int lim = (CAUSAL ? min(my_row, Lk - 1) : Lk - 1) - n0 - 4 * h;
-#pragma unroll
-      for (int nt = 0; nt < NT; nt++)
-#pragma unroll
-        for (int r = 0; r < 16; r++)
-        {
-          // branch-free select on the sign of (lim - index): compare-and-select would hold 64 lane masks
-          // in scalar registers at once
-          const int gone = (lim - (32 * nt + 8 * (r / 4) + (r % 4))) >> 31;
-          acc[nt][r] = (acc[nt][r] & ~gone) | (as_i(kNegInf) & gone);
-        }
-    }
-    // ---- row maximum of this tile, in score units ----
-    // The biased scores are positive floats (or -inf where masked), so their bit patterns order like
-    // signed integers: integer max3 needs no NaN canonicalisation.
-    mloc = kNegInf;
-#pragma unroll
-    for (int nt = 0; nt < NT; nt++) {
-      int mx = acc[nt][0];
-#pragma unroll
-      for (int r = 1; r < 16; r++) mx = max(mx, acc[nt][r]);
-      mloc = fmaxf(mloc, __builtin_fmaf(as_f(mx), sc[nt], -kBiasF * sc[nt]));
-    }
-  };
-
-  // ---- online softmax of the tile whose scores are in acc: pure VALU work ----
-  auto softmax = [&](int j) {
-    // next tile's K scales: requested first, consumed last
-    float kraw[NT];
-#pragma unroll
-    for (int nt = 0; nt < NT; nt++) kraw[nt] = ksc[min(((j + 1) * BN + 32 * nt) >> a.blkk_shift, nkblk - 1)];
-    const float mall = xchg32_max(mloc);
-    // lazy rescale: move the reference maximum only when it grew by more than TAU
-    if (__builtin_amdgcn_ballot_w64(mall > m_used + TAU) != 0) {
-      const float m_new = fmaxf(m_used, mall);
-      const float alpha = __builtin_amdgcn_exp2f(m_used - m_new);
-      lsum *= alpha;
-      if constexpr (MSUM) {
-#pragma unroll
-        for (int i = 0; i < 16; i++) osum[i] *= alpha;
-      }
-#pragma unroll
-      for (int dt = 0; dt < DTN; dt++)
-#pragma unroll
-        for (int i = 0; i < 16; i++) o[dt][i] *= alpha;
-      m_used = m_new;
-    }
-    // P = exp2(S - m) * 2^PSHIFT, packed straight into the B operand of the second MFMA
-    if constexpr (PV == 1) {
-#pragma unroll
-      for (int nt = 0; nt < NT; nt++) {
-        const float c = __builtin_fmaf(-kBiasF, sc[nt], PSHIFT - m_used);
-        float p[16];
-#pragma unroll
-        for (int r = 0; r < 16; r++) {
-          p[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(as_f(acc[nt][r]), sc[nt], c));
-          if constexpr (!MSUM) lsum += p[r];
-        }
-#pragma unroll
-        for (int q4 = 0; q4 < 4; q4++) {
-          // The packed probabilities of the whole tile (NT*4 dwords) take over the registers of acc[0],
-          // whose scores are consumed by then.  Both halves of each dword get written, so the 'old'
-          // operand is a don't-care: it is the destination register itself.
-          int d0 = __builtin_amdgcn_cvt_pk_fp8_f32(p[4 * q4], p[4 * q4 + 1], acc[0][4 * nt + q4], false);
-          acc[0][4 * nt + q4] = __builtin_amdgcn_cvt_pk_fp8_f32(p[4 * q4 + 2], p[4 * q4 + 3], d0, true);
-        }
-      }
-    } else {
-#pragma unroll
-      for (int nt = 0; nt < NT; nt++) {
-        const float c = __builtin_fmaf(-kBiasF, sc[nt], PSHIFT - m_used);
-#pragma unroll
-        for (int r = 0; r < 16; r++) {
-          float p = __builtin_amdgcn_exp2f(__builtin_fmaf(as_f(acc[nt][r]), sc[nt], c));
-          lsum += p;
-          ph[nt][r >> 3][r & 7] = (_Float16)p;
-        }
-      }
-    }
-#pragma unroll
-    for (int nt = 0; nt < NT; nt++) sc[nt] = qscale * kraw[nt];
-  };
-
-  // ---- O^T += V^T . P^T ----
-  auto pv = [&](int j) {
-    const uint8_t* vbuf = vslot(j);
-    if constexpr (PV == 1) {
-      constexpr int NV = (BN / 64) * DTN, VPF = 3;
-      auto vfrag = [&](int i) {
-        const uint8_t* vp0 = vbuf + ((i * 2) * 64 + lane) * 16;
-        v4i lo = *reinterpret_cast<const v4i*>(vp0);
-        v4i hi = *reinterpret_cast<const v4i*>(vp0 + 64 * 16);
-        return v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-      };
-      v8i vf[NV];
-#pragma unroll
-      for (int i = 0; i < VPF; i++) vf[i] = vfrag(i);
-#pragma unroll
-      for (int i = 0; i < NV; i++) {
-        const int kk = i / DTN, dt = i % DTN;
-        if (i + VPF < NV) vf[i + VPF] = vfrag(i + VPF);
-        v8i pb;
-#pragma unroll
-        for (int e = 0; e < 8; e++) pb[e] = acc[0][8 * kk + e];
-        if constexpr (MSUM) {
-          if (dt == 0) osum = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ones, pb, osum, 0, 0, 0, 0, 0, 0);
-        }
-        o[dt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vf[i], pb, o[dt], 0, 0, 0, 0, 0, 0);
-      }
-      __builtin_amdgcn_sched_group_barrier(0x100, 2 * VPF, 0);
-#pragma unroll
-      for (int i = 0; i < NV; i++) {
-        if (MSUM && i % DTN == 0) __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        if (i + VPF < NV) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-      }
-    } else {
-      constexpr int NV = (BN / 16) * DTN, VPF = 4;
-      auto vfrag = [&](int i) { return *reinterpret_cast<const v8h*>(vbuf + (i * 64 + lane) * 16); };
-      v8h vf[NV];
-#pragma unroll
-      for (int i = 0; i < VPF; i++) vf[i] = vfrag(i);
-#pragma unroll
-      for (int i = 0; i < NV; i++) {
-        const int k16 = i / DTN, dt = i % DTN;
-        if (i + VPF < NV) vf[i + VPF] = vfrag(i + VPF);
-        o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[i], ph[k16 >> 1][k16 & 1], o[dt], 0, 0, 0);
-      }
-      __builtin_amdgcn_sched_group_barrier(0x100, VPF, 0);
-#pragma unroll
-      for (int i = 0; i < NV; i++) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        if (i + VPF < NV) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      }
-    }
-  };
-
-  // ---- main loop: two groups of wavefronts half a tile apart ----
-  // A SIMD hosts one wavefront of each group.  In every phase one of them feeds the matrix pipe
-  // (P.V of its previous tile, then Q.K^T of its next tile) while the other runs the softmax of the
-  // tile in between on the vector ALU, and they swap at the next barrier: the two pipes of the SIMD
-  // are kept busy at the same time instead of taking turns.
-  //   phase 2j  : group 0: P.V(j-1), Q.K^T(j)      group 1: softmax(j-1)
-  //   phase 2j+1: group 0: softmax(j)              group 1: P.V(j-1), Q.K^T(j)
-  // K tile j is read in phases 2j and 2j+1, V tile j in phases 2j+2 and 2j+3; both are loaded one
-  // whole period before their first use, into the slot whose last reader finished a barrier ago.
-  if (ntiles > 0) {
-    const int grp = (w >> GSH) & 1;
-    const int wnt = wave_ntiles;
-    auto mfma_phase = [&](int j) {
-      if (j >= 1 && j - 1 < wnt) pv(j - 1);
-      if (j < wnt) { qk(j); rowmax(j); }
-    };
-    load_k(0);
-    load_scales(0);
-    auto even_barrier = [&](int j) {
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // my pieces of K(j) and V(j-1) have landed
-      lds_barrier();                                     // ... and everyone's; phase 2j-1 is over
-      if (j + 1 < ntiles) load_k(j + 1);
-      if (j < ntiles) load_v(j);
-    };
-    if (grp == 0) {
-      for (int j = 0; j <= ntiles; j++) {
-        even_barrier(j);
-        mfma_phase(j);
-        lds_barrier();
-        if (j < wnt) softmax(j);
-      }
-    } else {
-      for (int j = 0; j <= ntiles; j++) {
-        even_barrier(j);
-        if (j >= 1 && j - 1 < wnt) softmax(j - 1);
-        lds_barrier();
-        mfma_phase(j);
-      }
-    }
-  }
-
-  // ---- epilogue: O = O^T / l (* v_scale), LSE2 = m + log2(l) ----
-  if constexpr (MSUM) lsum = osum[0];   // already the full row sum (the MFMA contracts over both lane halves)
-  else lsum = xchg32_sum(lsum);
-  const float inv = lsum > 0.f ? 1.0f / lsum : 0.f;
-  if (my_row < Lq) {
-    if (a.lse && h == 0) a.lse[lseoff + my_row] = lsum > 0.f ? m_used + __builtin_amdgcn_logf(lsum) - PSHIFT : kNegInf;
-    const int64_t orow = ooff + (int64_t)my_row * a.o_sn;
-#pragma unroll
-    for (int dt = 0; dt < DTN; dt++) {
-#pragma unroll
-      for (int q4 = 0; q4 < 4; q4++) {
-        const int d = 32 * dt + 8 * q4 + 4 * h;
-        float f[4];
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-          f[i] = o[dt][4 * q4 + i] * inv;
-          if constexpr (PV == 1) f[i] *= a.vs[((int64_t)b * a.Hkv + kvh) * D + d + i];
-        }
-        u16 hv[4];
-#pragma unroll
-        for (int i = 0; i < 4; i++) hv[i] = a.out_bf16 ? f32_to_bf16(f[i]) : f32_to_f16(f[i]);
-        uint2 pkd = make_uint2((uint32_t)hv[0] | ((uint32_t)hv[1] << 16), (uint32_t)hv[2] | ((uint32_t)hv[3] << 16));
-        *reinterpret_cast<uint2*>(reinterpret_cast<u16*>(a.out) + orow + d) = pkd;
-      }
-    }
-  }
-}
 
 // ---------------------------------------------------------------------------------------------
 // Variable-length plan: block offsets per sequence and the cost-ordered tile list.
@@ -559,25 +70,11 @@ AttnConfig attn_config(int D, int pv, bool packed) {
   return c;
 }
 
-template <int D, int NW, int BN, int PV, bool CAUSAL, bool MSUM>
-static hipError_t launch_one(const AttnArgs& a, int grid, hipStream_t st) {
-  constexpr int VESZ = PV ? 1 : 2;
-  constexpr int smem = 2 * (BN * D + BN * D * VESZ);   // two K slots + two V slots
-  auto kern = attn_kernel<D, NW, BN, PV, CAUSAL, MSUM>;
-  static bool attr_done = false;
-  if (!attr_done) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
-    if (e != hipSuccess) return e;
-    attr_done = true;
-  }
-  kern<<<dim3(grid), dim3(NW * 64), smem, st>>>(a);
-  return hipGetLastError();
-}
-
 hipError_t launch_attn(const AttnArgs& a, int D, int pv, bool causal, int grid, hipStream_t st) {
   if (grid == 0) return hipSuccess;
+  if (a.mask) return launch_attn_masked(a, D, pv, grid, st);
   const bool msum = pv && a.lse == nullptr;   // row sums on the matrix pipe unless LSE is wanted
-#define SAGE_ATTN(DD, PVV, BNN, MS) (causal ? launch_one<DD, 8, BNN, PVV, true, MS>(a, grid, st) : launch_one<DD, 8, BNN, PVV, false, MS>(a, grid, st))
+#define SAGE_ATTN(DD, PVV, BNN, MS) (causal ? launch_one<DD, 8, BNN, PVV, true, MS, 0>(a, grid, st) : launch_one<DD, 8, BNN, PVV, false, MS, 0>(a, grid, st))
   if (D == 128) return pv ? (msum ? SAGE_ATTN(128, 1, 128, true) : SAGE_ATTN(128, 1, 128, false)) : SAGE_ATTN(128, 0, 64, false);
   return pv ? (msum ? SAGE_ATTN(64, 1, 128, true) : SAGE_ATTN(64, 1, 128, false)) : SAGE_ATTN(64, 0, 128, false);
 #undef SAGE_ATTN

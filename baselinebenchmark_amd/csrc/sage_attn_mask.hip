@@ -1,0 +1,15 @@
+// Fused attention kernel variants with an explicit attention mask (boolean or additive), the
+// rest of the forward() contract of backends/_hygon/ops/sageattention/sageattention_triton.py:92-105.
+// They live in their own translation unit so that the two sets of instantiations compile in parallel.
+#include "sage_attn_kernel.h"
+
+namespace sage {
+
+hipError_t launch_attn_masked(const AttnArgs& a, int D, int pv, int grid, hipStream_t st) {
+#define SAGE_ATTN_M(DD, PVV, BNN) (a.mask_kind == 1 ? launch_one<DD, 8, BNN, PVV, false, false, 1>(a, grid, st) : launch_one<DD, 8, BNN, PVV, false, false, 2>(a, grid, st))
+  if (D == 128) return pv ? SAGE_ATTN_M(128, 1, 128) : SAGE_ATTN_M(128, 0, 64);
+  return pv ? SAGE_ATTN_M(64, 1, 128) : SAGE_ATTN_M(64, 0, 128);
+#undef SAGE_ATTN_M
+}
+
+}  // namespace sage

@@ -16,6 +16,13 @@ struct QuantArgs {
   const int32_t* cu_seqlens;
   const int32_t* cu_blocks;
   int64_t scale_sh;
+  // optional row dot products (null dot_out: off): dotv is [B, H/dv_group, D] in the input dtype,
+  // dot_out is [B, H, L] (or [H, dot_total] for packed rows) fp32
+  const u16* dotv;
+  float* dot_out;
+  int64_t dv_sb, dv_sh;
+  int dv_group;
+  int dot_total;
 };
 
 struct ColStatArgs {
@@ -63,7 +70,13 @@ struct AttnArgs {
   const int32_t* tiles;
   int64_t qs_sh, ks_sh, panel_sh;
   int total_q;
-  int pp_split;  // 0: wavefront groups {0..NW/2-1 | NW/2..NW-1}; 1: even/odd wavefronts
+  // explicit mask (fixed-length mode only): [B, Hq, Sq, Skv] with element strides; kind 1 = bytes
+  // (non-zero keeps the key), 2 = fp32 added to the base-2 logits
+  const void* mask;
+  int mask_kind;
+  int64_t m_sb, m_sh, m_sm, m_sn;
+  float mask_mult;          // additive masks are scaled by this before they are added
+  const float* lse_offset;  // added to LSE2 per query row (same layout as lse) or null
 };
 
 struct AttnConfig { int nw, bn; };
@@ -76,6 +89,7 @@ hipError_t launch_prep_v(const PrepVArgs& a, int dtype, int pv, int max_panels, 
 
 AttnConfig attn_config(int D, int pv, bool packed);
 hipError_t launch_attn(const AttnArgs& a, int D, int pv, bool causal, int grid, hipStream_t st);
+hipError_t launch_attn_masked(const AttnArgs& a, int D, int pv, int grid, hipStream_t st);
 hipError_t launch_varlen_plan(const int32_t* cu_q, const int32_t* cu_k, int nseq, int total_q, int blkq, int blkk, int bm,
                               int bn, int causal, int32_t* plan, hipStream_t st);
 

@@ -40,10 +40,11 @@ __global__ void __launch_bounds__(256) quant_int8_kernel(QuantArgs a) {
   const int tr = tid / TPR, tc = tid % TPR;
 
   int L = a.L;
-  int64_t xbase, obase, sidx;
+  int64_t xbase, obase, sidx, dbase;
   if (a.cu_seqlens) {
     int s0 = a.cu_seqlens[b];
     L = a.cu_seqlens[b + 1] - s0;
+    dbase = (int64_t)h * a.dot_total + s0;
     xbase = (int64_t)s0 * a.x_sn + (int64_t)h * a.x_sh;
     obase = (int64_t)s0 * a.o_sn + (int64_t)h * a.o_sh;
     sidx = (int64_t)h * a.scale_sh + a.cu_blocks[b] + blkid;
@@ -51,6 +52,7 @@ __global__ void __launch_bounds__(256) quant_int8_kernel(QuantArgs a) {
     xbase = (int64_t)b * a.x_sb + (int64_t)h * a.x_sh;
     obase = (int64_t)b * a.o_sb + (int64_t)h * a.o_sh;
     sidx = ((int64_t)b * a.H + h) * ((L + a.blk - 1) / a.blk) + blkid;
+    dbase = ((int64_t)b * a.H + h) * L;
   }
   const int n0 = blkid * a.blk;
   if (n0 >= L) return;
@@ -71,12 +73,25 @@ __global__ void __launch_bounds__(256) quant_int8_kernel(QuantArgs a) {
     return x * a.mult;
   };
 
+  // Optional side output: the dot product of every (scaled) row with a per-(batch, kv-head) vector.
+  // The one-call pipeline uses it with the K mean to return the LSE of the unsmoothed logits.
+  const bool has_dot = a.dot_out != nullptr;
+  float dvv[16];
+  if (has_dot) {
+    const uint4* dp = reinterpret_cast<const uint4*>(a.dotv + (int64_t)b * a.dv_sb + (int64_t)(h / a.dv_group) * a.dv_sh + tc * 16);
+    uint4 raw2[2] = {dp[0], dp[1]};
+    const u16* p = reinterpret_cast<const u16*>(raw2);
+#pragma unroll
+    for (int i = 0; i < 16; i++) dvv[i] = to_f32<DT>(p[i]);
+  }
+
   uint4 raw[MAXP][2];
   float amax = 0.f;
 #pragma unroll
   for (int p = 0; p < MAXP; p++) {
     int r = p * RPP + tr;
     raw[p][0] = raw[p][1] = make_uint4(0, 0, 0, 0);
+    float dsum = 0.f;
     if (r < rows) {
       const uint4* src = reinterpret_cast<const uint4*>(a.x + xbase + (int64_t)(n0 + r) * a.x_sn + tc * 16);
       raw[p][0] = src[0];
@@ -84,6 +99,15 @@ __global__ void __launch_bounds__(256) quant_int8_kernel(QuantArgs a) {
       const u16* e = reinterpret_cast<const u16*>(raw[p]);
 #pragma unroll
       for (int i = 0; i < 16; i++) amax = fmaxf(amax, fabsf(value(e[i], i)));
+      if (has_dot) {
+#pragma unroll
+        for (int i = 0; i < 16; i++) dsum = __builtin_fmaf(value(e[i], i), dvv[i], dsum);
+      }
+    }
+    if (has_dot) {   // uniform branch; the TPR lanes of a row are neighbours inside one wavefront
+#pragma unroll
+      for (int o = 1; o < TPR; o <<= 1) dsum += __shfl_xor(dsum, o);
+      if (r < rows && tc == 0) a.dot_out[dbase + n0 + r] = dsum;
     }
   }
   __shared__ float wmax[4];

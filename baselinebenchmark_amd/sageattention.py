@@ -167,6 +167,32 @@ def _pv(pv_mode) -> int:
     raise ValueError(f"pv_mode {pv_mode!r} is not 'fp16' or 'fp8'")
 
 
+def _mask_args(attn_mask, B, Hq, Sq, Skv, device):
+    """Validate an explicit mask and return (tensor kept alive, kind, element strides).
+
+    Boolean masks keep the keys that are True; any other dtype is an additive bias and is read as
+    fp32 (sageattention_triton.py:180-186, :92-105).  The mask must be broadcastable to
+    [B, Hq, Sq, Skv]; broadcast dimensions are passed with stride 0, nothing is materialised.
+    """
+    if not isinstance(attn_mask, torch.Tensor):
+        raise TypeError("attn_mask must be a tensor")
+    if not attn_mask.is_cuda or attn_mask.device != device:
+        raise ValueError("attn_mask must be on the same device as q")
+    if attn_mask.ndim > 4:
+        raise ValueError("attn_mask must have at most 4 dimensions")
+    if attn_mask.dtype == torch.bool:
+        kind, m = 1, attn_mask
+    elif attn_mask.dtype.is_floating_point:
+        kind, m = 2, attn_mask if attn_mask.dtype == torch.float32 else attn_mask.float()
+    else:
+        raise TypeError("attn_mask must be boolean or floating point")
+    try:
+        m = m.expand(B, Hq, Sq, Skv)
+    except RuntimeError as exc:
+        raise ValueError(f"attn_mask of shape {tuple(attn_mask.shape)} does not broadcast to {(B, Hq, Sq, Skv)}") from exc
+    return m, kind, m.stride()
+
+
 # ------------------------------------------------------------------------------------------------
 # attention on quantised operands
 # ------------------------------------------------------------------------------------------------
@@ -180,6 +206,8 @@ def forward(q, k, v, q_scale, k_scale, tensor_layout="HND", attn_mask=None, outp
     keywords (maxnreg, block_m, num_warps, num_stages, backend) are accepted and ignored as in
     sageattention_triton.py:169.  Additions: ``BLKQ``/``BLKK`` name the scale blocks when they are
     not the reference's 128/64, ``is_causal`` and ``pv_mode`` ("fp16" | "fp8").
+    ``attn_mask``: boolean (True keeps the key) or additive bias on the base-2 logits, broadcastable
+    to [B, Hq, Sq, Skv] (sageattention_triton.py:92-105); not combinable with ``is_causal``.
     ``lse`` is base 2 (sageattention_triton.py:127-129) and an empty tensor unless requested.
     """
     for name, t in (("q", q), ("k", k)):
@@ -192,8 +220,8 @@ def forward(q, k, v, q_scale, k_scale, tensor_layout="HND", attn_mask=None, outp
         raise NotImplementedError("output_dtype must be FP16 or BF16")
     if maxnreg is not None and maxnreg <= 0:
         raise ValueError("maxnreg must be positive")
-    if attn_mask is not None:
-        raise NotImplementedError("attn_mask is not supported by the MI355X kernel (use is_causal)")
+    if attn_mask is not None and is_causal:
+        raise NotImplementedError("attn_mask cannot be combined with is_causal")
     if q.ndim != 4 or k.ndim != 4:
         raise ValueError("q, k, and v must be rank-4 tensors")
     B, Hq, Sq, D, qsb, qsh, qsn = _layout(q, tensor_layout)
@@ -216,10 +244,20 @@ def forward(q, k, v, q_scale, k_scale, tensor_layout="HND", attn_mask=None, outp
     if q_scale.device != q.device or k_scale.device != q.device or k.device != q.device or v.device != q.device:
         raise ValueError("all tensors must be on the same device")
     pv = _pv(pv_mode)
+    mask_info = _mask_args(attn_mask, B, Hq, Sq, Skv, q.device) if attn_mask is not None else None
     panels, v_scale = prepare_v(v, tensor_layout, pv)
     out = torch.empty(q.shape, device=q.device, dtype=output_dtype)
     _, _, _, _, osb, osh, osn = _layout(out, tensor_layout)
     lse = torch.empty((B, Hq, Sq), device=q.device, dtype=torch.float32) if return_lse else torch.empty(0, device=q.device)
+    if mask_info is not None:
+        m, kind, ms = mask_info
+        check(lib().sage_attn_fwd_masked(_ptr(q), _ptr(k), _ptr(panels), _ptr(q_scale.contiguous()),
+                                         _ptr(k_scale.contiguous()), _ptr(v_scale), _ptr(out),
+                                         _ptr(lse if return_lse else None),
+                                         B, Hq, Hkv, Sq, Skv, D, qsb, qsh, qsn, ksb, ksh, ksn, osb, osh, osn,
+                                         BLKQ, BLKK, pv, _dt(output_dtype), _ptr(m), kind, ms[0], ms[1], ms[2], ms[3],
+                                         _stream(q)))
+        return out, lse
     check(lib().sage_attn_fwd(_ptr(q), _ptr(k), _ptr(panels), _ptr(q_scale.contiguous()), _ptr(k_scale.contiguous()),
                               _ptr(v_scale), _ptr(out), _ptr(lse if return_lse else None),
                               B, Hq, Hkv, Sq, Skv, D, qsb, qsh, qsn, ksb, ksh, ksn, osb, osh, osn,
@@ -233,11 +271,14 @@ def forward(q, k, v, q_scale, k_scale, tensor_layout="HND", attn_mask=None, outp
 # ------------------------------------------------------------------------------------------------
 @torch.no_grad()
 def sageattn(q, k, v, tensor_layout="HND", is_causal=False, sm_scale=None, smooth_k=True, pv_mode="fp16",
-             BLKQ=128, BLKK=64, return_lse=False, qk_quant_dtype="int8", quant_recipe=None, **kwargs):
-    """Quantise + attend in one call: out = softmax(q k^T * sm_scale [causal]) v.
+             BLKQ=128, BLKK=64, return_lse=False, qk_quant_dtype="int8", quant_recipe=None, attn_mask=None, **kwargs):
+    """Quantise + attend in one call: out = softmax(q k^T * sm_scale [causal | + attn_mask]) v.
 
     Returns ``out`` (q's shape and dtype), or ``(out, lse)`` with ``return_lse=True`` where lse is
-    the natural-log LSE of the *smoothed* logits (q.(k - mean_k)) * sm_scale.
+    the natural-log log-sum-exp of ``sm_scale * q k^T (+ mask)`` for the ORIGINAL k: what K smoothing
+    removes from the logits is added back (checked as in test_sage_attention_mate.py:171-178).
+    ``attn_mask``: boolean (True keeps) or additive in natural-log units, broadcastable to
+    [B, Hq, Sq, Skv]; not combinable with ``is_causal``.
     """
     if qk_quant_dtype != "int8":
         raise NotImplementedError("only INT8 Q/K quantisation is implemented")
@@ -264,10 +305,20 @@ def sageattn(q, k, v, tensor_layout="HND", is_causal=False, sm_scale=None, smoot
     lse = torch.empty((B, Hq, Sq), device=q.device, dtype=torch.float32) if return_lse else None
     ws_bytes = lib().sage_sageattn_workspace_bytes(B, Hq, Hkv, Sq, Skv, D, BLKQ, BLKK, pv, 0, 0, 0)
     ws = torch.empty(max(ws_bytes, 256), device=q.device, dtype=torch.uint8)
-    check(lib().sage_sageattn(_ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _ptr(ws), ws_bytes,
-                              B, Hq, Hkv, Sq, Skv, D, qsb, qsh, qsn, ksb, ksh, ksn, vsb, vsh, vsn, osb, osh, osn,
-                              _dt(q.dtype), BLKQ, BLKK, float(D ** -0.5 if sm_scale is None else sm_scale),
-                              int(bool(is_causal)), int(bool(smooth_k)), pv, None, None, 0, 0, _stream(q)))
+    if attn_mask is not None:
+        if is_causal:
+            raise NotImplementedError("attn_mask cannot be combined with is_causal")
+        m, kind, ms = _mask_args(attn_mask, B, Hq, Sq, Skv, q.device)
+        check(lib().sage_sageattn_masked(_ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _ptr(ws), ws_bytes,
+                                         B, Hq, Hkv, Sq, Skv, D, qsb, qsh, qsn, ksb, ksh, ksn, vsb, vsh, vsn, osb, osh, osn,
+                                         _dt(q.dtype), BLKQ, BLKK, float(D ** -0.5 if sm_scale is None else sm_scale),
+                                         0, int(bool(smooth_k)), pv, None, None, 0, 0,
+                                         _ptr(m), kind, ms[0], ms[1], ms[2], ms[3], _stream(q)))
+    else:
+        check(lib().sage_sageattn(_ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _ptr(ws), ws_bytes,
+                                  B, Hq, Hkv, Sq, Skv, D, qsb, qsh, qsn, ksb, ksh, ksn, vsb, vsh, vsn, osb, osh, osn,
+                                  _dt(q.dtype), BLKQ, BLKK, float(D ** -0.5 if sm_scale is None else sm_scale),
+                                  int(bool(is_causal)), int(bool(smooth_k)), pv, None, None, 0, 0, _stream(q)))
     if return_lse:
         return out, lse * 0.6931471805599453
     return out

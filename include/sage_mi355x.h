@@ -38,6 +38,10 @@ extern "C" {
 #define SAGE_PV_FP16 0 /* P and V in fp16, fp32 accumulate (the reference's _attention_kernel)   */
 #define SAGE_PV_FP8 1  /* P and V in fp8-e4m3fn, fp32 accumulate, per-channel V scale            */
 
+/* explicit attention masks (sageattention_triton.py:180-186: MASK_KIND 1 / 2) */
+#define SAGE_MASK_BOOL 1     /* bytes; non-zero = the key is visible (torch.bool)                */
+#define SAGE_MASK_ADDITIVE 2 /* fp32 bias added to the logits                                    */
+
 /* Rows of K/V covered by one V panel (see sage_prep_v). */
 #define SAGE_PANEL_ROWS 128
 
@@ -147,6 +151,28 @@ int sage_attn_fwd(const int8_t* q, const int8_t* k, const void* v_panels,
                   sage_stream_t stream);
 
 /*
+ * The same with an explicit mask: the attn_mask argument of forward
+ * (sageattention_triton.py:167-168, :92-105; exercised by
+ * backends/_hygon/test/sageattention/test_sageattention_hip.py:40-45, :65-66).
+ * attn_mask is [B, Hq, Sq, Skv] addressed with ELEMENT strides (m_sb, m_sh, m_sm, m_sn; 0 broadcasts):
+ *   SAGE_MASK_BOOL     : logits of keys whose byte is 0 become -inf;
+ *   SAGE_MASK_ADDITIVE : the fp32 value is added to the base-2 logits (q_scale already holds
+ *                        sm_scale*log2(e), so the bias is in those units, as in the reference).
+ * A row with no visible key yields out = 0 and LSE2 = -inf.  No causal flag and no packed mode here.
+ */
+int sage_attn_fwd_masked(const int8_t* q, const int8_t* k, const void* v_panels,
+                         const float* q_scale, const float* k_scale, const float* v_scale,
+                         void* out, float* lse,
+                         int B, int Hq, int Hkv, int Sq, int Skv, int D,
+                         int64_t q_sb, int64_t q_sh, int64_t q_sn,
+                         int64_t k_sb, int64_t k_sh, int64_t k_sn,
+                         int64_t o_sb, int64_t o_sh, int64_t o_sn,
+                         int blkq, int blkk, int pv_mode, int out_dtype,
+                         const void* attn_mask, int mask_kind,
+                         int64_t m_sb, int64_t m_sh, int64_t m_sm, int64_t m_sn,
+                         sage_stream_t stream);
+
+/*
  * One-call pipeline behind sageattn(q, k, v, tensor_layout, is_causal, sm_scale, ...) -- the
  * entry point exercised at backends/_metax/benchmarks/sage_attention/benchmark.py:29 and
  * backends/_mthreads/benchmarks/sage_attention_benchmark_compare.py:300-313:
@@ -155,6 +181,8 @@ int sage_attn_fwd(const int8_t* q, const int8_t* k, const void* v_panels,
  * smooth_k != 0 subtracts the per-channel K mean.  sm_scale <= 0 selects head_dim^-0.5; the Q
  * multiplier is (float)(sm_scale * 1.44269504), the double product of quant_per_block.py:87.  Packed mode as in sage_attn_fwd
  * (cu_seqlens_* != NULL; total_q/total_k = packed row counts).
+ * lse (may be NULL) receives the base-2 log-sum-exp of the logits of the ORIGINAL k: with smooth_k the
+ * term q . k_mean that smoothing removed from every logit of a row is added back.
  */
 size_t sage_sageattn_workspace_bytes(int B, int Hq, int Hkv, int Sq, int Skv, int D,
                                      int blkq, int blkk, int pv_mode, int total_q, int total_k,
@@ -171,6 +199,27 @@ int sage_sageattn(const void* q, const void* k, const void* v, void* out, float*
                   const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
                   int total_q, int total_k,
                   sage_stream_t stream);
+
+/*
+ * sageattn with an explicit mask, the call of
+ * backends/_mthreads/tests/test_sage_attention_mate.py:186-208 (attn_mask keyword) checked against
+ * softmax(sm_scale * q.k^T + mask) at :171-178: here the additive mask is in NATURAL-log units on top
+ * of sm_scale * q.k^T (it is multiplied by log2(e) internally); boolean masks as in
+ * sage_attn_fwd_masked.  attn_mask == NULL makes it identical to sage_sageattn.
+ */
+int sage_sageattn_masked(const void* q, const void* k, const void* v, void* out, float* lse,
+                         void* workspace, size_t workspace_bytes,
+                         int B, int Hq, int Hkv, int Sq, int Skv, int D,
+                         int64_t q_sb, int64_t q_sh, int64_t q_sn,
+                         int64_t k_sb, int64_t k_sh, int64_t k_sn,
+                         int64_t v_sb, int64_t v_sh, int64_t v_sn,
+                         int64_t o_sb, int64_t o_sh, int64_t o_sn,
+                         int dtype, int blkq, int blkk, double sm_scale, int is_causal, int smooth_k,
+                         int pv_mode, const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+                         int total_q, int total_k,
+                         const void* attn_mask, int mask_kind,
+                         int64_t m_sb, int64_t m_sh, int64_t m_sm, int64_t m_sn,
+                         sage_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -61,8 +61,14 @@ def test_forward_contract():
         sa.forward(q, k, v, qs, ks, output_dtype=torch.float32)
     with pytest.raises(ValueError):
         sa.forward(q, k, v, qs, ks, maxnreg=0)
-    with pytest.raises(NotImplementedError):
+    with pytest.raises(NotImplementedError):   # an explicit mask and the causal flag exclude each other
+        sa.forward(q, k, v, qs, ks, attn_mask=fake(1, 4, 128, 128, dtype=torch.bool), is_causal=True)
+    with pytest.raises(ValueError):             # mask on another device
         sa.forward(q, k, v, qs, ks, attn_mask=torch.ones(1, 4, 128, 128, dtype=torch.bool))
+    with pytest.raises(ValueError):             # not broadcastable to [B, Hq, Sq, Skv]
+        sa.forward(q, k, v, qs, ks, attn_mask=fake(1, 4, 128, 100, dtype=torch.bool))
+    with pytest.raises(TypeError):              # neither boolean nor floating point
+        sa.forward(q, k, v, qs, ks, attn_mask=fake(1, 4, 128, 128, dtype=torch.int32))
     with pytest.raises(ValueError):
         sa.forward(q, k, fake(1, 2, 64, 64), qs, ks)  # v length differs
     with pytest.raises(ValueError):
