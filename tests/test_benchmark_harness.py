@@ -1,0 +1,65 @@
+"""The benchmark harness: shape table, options and statistics on the CPU; one tiny run on the GPU.
+
+What it mirrors: the 20-shape table, the custom-shape options, the validation rules and the ops formula of
+backends/_enflame/benchmarks/sage_attention_native_benchmark.py:70-78, :158-198, :447-455.
+"""
+import json
+
+import pytest
+
+from baselinebenchmark_amd.benchmarks import sage_attention_benchmark as bench
+
+
+def test_default_table_is_the_references_20_shapes_in_its_order():
+    args = bench.build_parser().parse_args([])
+    shapes = bench.configs(args)
+    assert len(shapes) == 20 and len(set(shapes)) == 20
+    assert shapes[0] == (1, 1024, 32, 32, 64, "float16")
+    assert shapes[4] == (1, 16384, 32, 32, 64, "float16")
+    assert shapes[5] == (1, 1024, 32, 32, 128, "float16")
+    assert shapes[10] == (1, 1024, 32, 32, 64, "bfloat16")
+    assert shapes[-1] == (1, 16384, 32, 32, 128, "bfloat16")
+    assert {(b, t) for b, t, *_ in shapes} == {(1, 1024), (4, 1024), (1, 4096), (1, 8192), (1, 16384)}
+
+
+def test_custom_shapes_and_validation():
+    p = bench.build_parser()
+    args = p.parse_args(["--custom-shapes", "--batch-size", "2", "--num-heads", "32", "--num-kv-heads", "8", "--head-dim", "128",
+                         "--seq-lens", "512", "2048", "--dtype", "bfloat16"])
+    bench.validate(args)
+    assert bench.configs(args) == [(2, 512, 32, 8, 128, "bfloat16"), (2, 2048, 32, 8, 128, "bfloat16")]
+    with pytest.raises(ValueError):
+        bench.validate(p.parse_args(["--custom-shapes", "--num-heads", "6", "--num-kv-heads", "4"]))
+    with pytest.raises(ValueError):
+        bench.validate(p.parse_args(["--rep", "0"]))
+    with pytest.raises(ValueError):
+        bench.validate(p.parse_args(["--atol", "-1"]))
+    with pytest.raises(SystemExit):
+        p.parse_args(["--head-dim", "96"])
+
+
+def test_ops_formula_and_statistics():
+    assert bench.effective_ops(2, 32, 16384, 128, True) == 4398046511104.0      # BASELINE config 2
+    assert bench.effective_ops(1, 32, 1024, 64, False) == 4 * 32 * 1024 * 1024 * 64
+    s = bench.summarise([3.0, 1.0, 2.0, 100.0, 4.0])
+    assert s["samples"] == 5 and s["median_ms"] == 3.0 and s["p99_ms"] == 100.0 and s["min_ms"] == 1.0 and s["mean_ms"] == 22.0
+    s = bench.summarise([float(i) for i in range(1, 201)])
+    assert s["p99_ms"] == 198.0 and s["median_ms"] == 100.5
+
+
+@pytest.mark.gpu
+@pytest.mark.sage_attention
+def test_tiny_run_gates_then_times_and_writes_a_result_file(tmp_path):
+    args = bench.build_parser().parse_args(["--custom-shapes", "--path", "both", "--batch-size", "1", "--num-heads", "4",
+                                            "--num-kv-heads", "2", "--head-dim", "64", "--seq-lens", "256", "--warmup", "1",
+                                            "--rep", "3", "--results-dir", str(tmp_path)])
+    rows = bench.benchmark(args)
+    assert [r["path"] for r in rows] == ["core", "e2e"]
+    for r in rows:
+        assert r["status"] == "PASS" and float(r["latency_ms"]) > 0 and float(r["gate_max_abs"]) < 3e-2 and r["samples"] == 3
+    files = list(tmp_path.glob("sage_attention_mi355x_*.json"))
+    assert len(files) == 1
+    doc = json.loads(files[0].read_text())
+    for key in ("backend", "device", "operator", "framework_version", "driver_version", "commit", "cases", "tolerance"):
+        assert key in doc
+    assert doc["cases"][0]["shape"] == [1, 4, 256, 64] and doc["cases"][0]["warmup"] == 1
