@@ -32,6 +32,7 @@ inline size_t align_up(size_t x, size_t a = 256) { return (x + a - 1) / a * a; }
 
 bool valid_blk_quant(int blk) { return blk == 16 || blk == 32 || blk == 64 || blk == 128; }
 bool valid_blk_attn(int blk) { return blk == 32 || blk == 64 || blk == 128; }
+bool valid_blkk_attn(int blk) { return blk == 16 || valid_blk_attn(blk); }
 int ilog2(int x) { int r = 0; while ((1 << r) < x) r++; return r; }
 
 int check_common(int B, int H, int L, int D, int dtype) {
@@ -202,8 +203,9 @@ int attn_impl(const int8_t* q, const int8_t* k, const void* v_panels, const floa
   if (Hkv <= 0 || Hq % Hkv) return fail(SAGE_EINVAL, "query heads (%d) must be divisible by KV heads (%d)", Hq, Hkv);
   if (Skv < 0) return fail(SAGE_EINVAL, "negative kv length");
   if (pv_mode != SAGE_PV_FP16 && pv_mode != SAGE_PV_FP8) return fail(SAGE_EINVAL, "pv_mode %d unknown", pv_mode);
-  if (!valid_blk_attn(blkq) || !valid_blk_attn(blkk))
-    return fail(SAGE_ENOTIMPL, "attention needs scale blocks of 32, 64 or 128 rows (got %d/%d)", blkq, blkk);
+  if (!valid_blk_attn(blkq) || !valid_blkk_attn(blkk))
+    return fail(SAGE_ENOTIMPL, "attention needs Q scale blocks of 32/64/128 rows and K scale blocks of 16/32/64/128 rows (got %d/%d)", blkq, blkk);
+  if (blkk == 16 && mask.ptr) return fail(SAGE_ENOTIMPL, "K scale blocks of 16 rows cannot be combined with an explicit mask");
   if (B == 0 || Hq == 0 || Sq == 0) return SAGE_OK;
   if (!q || !k || !v_panels || !q_scale || !k_scale || !out) return fail(SAGE_EINVAL, "null tensor pointer");
   if (pv_mode == SAGE_PV_FP8 && !v_scale) return fail(SAGE_EINVAL, "fp8 P.V needs v_scale");
@@ -337,8 +339,8 @@ int sage_sageattn_masked(const void* q, const void* k, const void* v, void* out,
                          int64_t m_sm, int64_t m_sn, sage_stream_t stream) {
   if (int rc = check_common(B, Hq, Sq, D, dtype)) return rc;
   if (Hkv <= 0 || Hq % Hkv) return fail(SAGE_EINVAL, "query heads (%d) must be divisible by KV heads (%d)", Hq, Hkv);
-  if (!valid_blk_attn(blkq) || !valid_blk_attn(blkk))
-    return fail(SAGE_ENOTIMPL, "scale blocks must be 32, 64 or 128 rows (got %d/%d)", blkq, blkk);
+  if (!valid_blk_attn(blkq) || !valid_blkk_attn(blkk))
+    return fail(SAGE_ENOTIMPL, "Q scale blocks must be 32/64/128 rows and K scale blocks 16/32/64/128 rows (got %d/%d)", blkq, blkk);
   if (pv_mode != SAGE_PV_FP16 && pv_mode != SAGE_PV_FP8) return fail(SAGE_EINVAL, "pv_mode %d unknown", pv_mode);
   const int varlen = cu_seqlens_q != nullptr;
   if (varlen && !cu_seqlens_k) return fail(SAGE_EINVAL, "packed mode needs cu_seqlens_k");

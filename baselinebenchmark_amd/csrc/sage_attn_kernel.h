@@ -88,7 +88,8 @@ __device__ inline int kswz(int n) {
 
 // MASK: 0 none, 1 boolean keep-mask (bytes), 2 additive fp32 bias in base-2 score units
 // (sageattention_triton.py:92-105), both [B, Hq, Sq, Skv] with element strides.
-template <int D, int NW, int BN, int PV, bool CAUSAL, bool MSUM, int MASK>
+// KSUB: K scale blocks per 32 keys (1 for blocks of 32/64/128 keys, 2 for blocks of 16 keys).
+template <int D, int NW, int BN, int PV, bool CAUSAL, bool MSUM, int MASK, int KSUB = 1>
 __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
   constexpr int GSH = SAGE_GSH;   // which bit of the wavefront index picks the group
   constexpr int BM = NW * 32;
@@ -246,7 +247,11 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
   // State that crosses phases: the raw scores of the tile in flight, its row maximum and scales, and
   // the probabilities packed as the B operand of the second MFMA.
   v16i acc[NT];
-  float sc[NT];
+  // q_scale * k_scale per K scale block of the tile; in the accumulator layout register r of a 32-key
+  // group holds keys 8*(r/4) + 4*h + r%4, so registers 0-7 belong to the first 16 keys and 8-15 to the rest.
+  constexpr int NSC = NT * KSUB;
+  float sc[NSC];
+  auto sci = [](int nt, int r) { return KSUB == 2 ? 2 * nt + r / 8 : nt; };
   float mloc = kNegInf;
   v8h ph[NT][2];      // fp16 mode
 
@@ -283,7 +288,7 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
   // load in flight while K/V fragments are being read would force every LDS wait to drain the queue.
   auto load_scales = [&](int j) {
 #pragma unroll
-    for (int nt = 0; nt < NT; nt++) sc[nt] = qscale * ksc[min((j * BN + 32 * nt) >> a.blkk_shift, nkblk - 1)];
+    for (int i = 0; i < NSC; i++) sc[i] = qscale * ksc[min((j * BN + (32 / KSUB) * i) >> a.blkk_shift, nkblk - 1)];
   };
 
   auto rowmax = [&](int j) {
@@ -295,11 +300,10 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
       mloc = kNegInf;
 #pragma unroll
       for (int nt = 0; nt < NT; nt++) {
-        const float off = -kBiasF * sc[nt];
 #pragma unroll
         for (int r = 0; r < 16; r++) {
           const int n = n0 + 32 * nt + 8 * (r / 4) + 4 * h + (r % 4);
-          float sv = __builtin_fmaf(as_f(acc[nt][r]), sc[nt], off);
+          float sv = __builtin_fmaf(as_f(acc[nt][r]), sc[sci(nt, r)], -kBiasF * sc[sci(nt, r)]);
           const int64_t mi = mrow + (int64_t)min(n, Lk - 1) * a.m_sn;
           if constexpr (MASK == 1) sv = reinterpret_cast<const uint8_t*>(a.mask)[mi] ? sv : kNegInf;
           else sv = __builtin_fmaf(reinterpret_cast<const float*>(a.mask)[mi], a.mask_mult, sv);
@@ -331,19 +335,23 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
     mloc = kNegInf;
 #pragma unroll
     for (int nt = 0; nt < NT; nt++) {
-      int mx = acc[nt][0];
 #pragma unroll
-      for (int r = 1; r < 16; r++) mx = max(mx, acc[nt][r]);
-      mloc = fmaxf(mloc, __builtin_fmaf(as_f(mx), sc[nt], -kBiasF * sc[nt]));
+      for (int sub = 0; sub < KSUB; sub++) {
+        constexpr int RS = 16 / KSUB;
+        int mx = acc[nt][sub * RS];
+#pragma unroll
+        for (int r = 1; r < RS; r++) mx = max(mx, acc[nt][sub * RS + r]);
+        mloc = fmaxf(mloc, __builtin_fmaf(as_f(mx), sc[nt * KSUB + sub], -kBiasF * sc[nt * KSUB + sub]));
+      }
     }
   };
 
   // ---- online softmax of the tile whose scores are in acc: pure VALU work ----
   auto softmax = [&](int j) {
     // next tile's K scales: requested first, consumed last
-    float kraw[NT];
+    float kraw[NSC];
 #pragma unroll
-    for (int nt = 0; nt < NT; nt++) kraw[nt] = ksc[min(((j + 1) * BN + 32 * nt) >> a.blkk_shift, nkblk - 1)];
+    for (int i = 0; i < NSC; i++) kraw[i] = ksc[min(((j + 1) * BN + (32 / KSUB) * i) >> a.blkk_shift, nkblk - 1)];
     const float mall = xchg32_max(mloc);
     // lazy rescale: move the reference maximum only when it grew by more than TAU
     if (__builtin_amdgcn_ballot_w64(mall > m_used + TAU) != 0) {
@@ -364,12 +372,16 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
     if constexpr (PV == 1) {
 #pragma unroll
       for (int nt = 0; nt < NT; nt++) {
-        const float c = MASK ? PSHIFT - m_used : __builtin_fmaf(-kBiasF, sc[nt], PSHIFT - m_used);
-        const float mul = MASK ? 1.0f : sc[nt];   // masked variants already hold scores
+        float c[KSUB], mul[KSUB];
+#pragma unroll
+        for (int sub = 0; sub < KSUB; sub++) {
+          c[sub] = MASK ? PSHIFT - m_used : __builtin_fmaf(-kBiasF, sc[nt * KSUB + sub], PSHIFT - m_used);
+          mul[sub] = MASK ? 1.0f : sc[nt * KSUB + sub];   // masked variants already hold scores
+        }
         float p[16];
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-          p[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(as_f(acc[nt][r]), mul, c));
+          p[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(as_f(acc[nt][r]), mul[KSUB == 2 ? r / 8 : 0], c[KSUB == 2 ? r / 8 : 0]));
           if constexpr (!MSUM) lsum += p[r];
         }
 #pragma unroll
@@ -384,18 +396,22 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
     } else {
 #pragma unroll
       for (int nt = 0; nt < NT; nt++) {
-        const float c = MASK ? PSHIFT - m_used : __builtin_fmaf(-kBiasF, sc[nt], PSHIFT - m_used);
-        const float mul = MASK ? 1.0f : sc[nt];
+        float c[KSUB], mul[KSUB];
+#pragma unroll
+        for (int sub = 0; sub < KSUB; sub++) {
+          c[sub] = MASK ? PSHIFT - m_used : __builtin_fmaf(-kBiasF, sc[nt * KSUB + sub], PSHIFT - m_used);
+          mul[sub] = MASK ? 1.0f : sc[nt * KSUB + sub];
+        }
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-          float p = __builtin_amdgcn_exp2f(__builtin_fmaf(as_f(acc[nt][r]), mul, c));
+          float p = __builtin_amdgcn_exp2f(__builtin_fmaf(as_f(acc[nt][r]), mul[KSUB == 2 ? r / 8 : 0], c[KSUB == 2 ? r / 8 : 0]));
           lsum += p;
           ph[nt][r >> 3][r & 7] = (_Float16)p;
         }
       }
     }
 #pragma unroll
-    for (int nt = 0; nt < NT; nt++) sc[nt] = qscale * kraw[nt];
+    for (int i = 0; i < NSC; i++) sc[i] = qscale * kraw[i];
   };
 
   // ---- O^T += V^T . P^T ----
@@ -526,11 +542,11 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
 }
 
 
-template <int D, int NW, int BN, int PV, bool CAUSAL, bool MSUM, int MASK>
+template <int D, int NW, int BN, int PV, bool CAUSAL, bool MSUM, int MASK, int KSUB = 1>
 static hipError_t launch_one(const AttnArgs& a, int grid, hipStream_t st) {
   constexpr int VESZ = PV ? 1 : 2;
   constexpr int smem = 2 * (BN * D + BN * D * VESZ);   // two K slots + two V slots
-  auto kern = attn_kernel<D, NW, BN, PV, CAUSAL, MSUM, MASK>;
+  auto kern = attn_kernel<D, NW, BN, PV, CAUSAL, MSUM, MASK, KSUB>;
   static bool attr_done = false;
   if (!attr_done) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem);

@@ -1,6 +1,8 @@
 // Fused attention kernel variants with an explicit attention mask (boolean or additive), the
 // rest of the forward() contract of backends/_hygon/ops/sageattention/sageattention_triton.py:92-105.
-// They live in their own translation unit so that the two sets of instantiations compile in parallel.
+// Also here: the variants for K scale blocks of 16 keys (the external MATE recipe (128, 16),
+// backends/_mthreads/benchmarks/sage_attention_benchmark_compare.py:93).
+// They live in their own translation unit so that the sets of instantiations compile in parallel.
 #include "sage_attn_kernel.h"
 
 namespace sage {
@@ -10,6 +12,13 @@ hipError_t launch_attn_masked(const AttnArgs& a, int D, int pv, int grid, hipStr
   if (D == 128) return pv ? SAGE_ATTN_M(128, 1, 128) : SAGE_ATTN_M(128, 0, 64);
   return pv ? SAGE_ATTN_M(64, 1, 128) : SAGE_ATTN_M(64, 0, 128);
 #undef SAGE_ATTN_M
+}
+
+hipError_t launch_attn_k16(const AttnArgs& a, int D, int pv, bool causal, int grid, hipStream_t st) {
+#define SAGE_ATTN_K(DD, PVV, BNN) (causal ? launch_one<DD, 8, BNN, PVV, true, false, 0, 2>(a, grid, st) : launch_one<DD, 8, BNN, PVV, false, false, 0, 2>(a, grid, st))
+  if (D == 128) return pv ? SAGE_ATTN_K(128, 1, 128) : SAGE_ATTN_K(128, 0, 64);
+  return pv ? SAGE_ATTN_K(64, 1, 128) : SAGE_ATTN_K(64, 0, 128);
+#undef SAGE_ATTN_K
 }
 
 }  // namespace sage

@@ -90,6 +90,7 @@ hipError_t launch_prep_v(const PrepVArgs& a, int dtype, int pv, int max_panels, 
 AttnConfig attn_config(int D, int pv, bool packed);
 hipError_t launch_attn(const AttnArgs& a, int D, int pv, bool causal, int grid, hipStream_t st);
 hipError_t launch_attn_masked(const AttnArgs& a, int D, int pv, int grid, hipStream_t st);
+hipError_t launch_attn_k16(const AttnArgs& a, int D, int pv, bool causal, int grid, hipStream_t st);
 hipError_t launch_varlen_plan(const int32_t* cu_q, const int32_t* cu_k, int nseq, int total_q, int blkq, int blkk, int bm,
                               int bn, int causal, int32_t* plan, hipStream_t st);
 

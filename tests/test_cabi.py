@@ -77,7 +77,8 @@ def test_attn_argument_errors(sage_lib):
                                       NULL, NULL, NULL, 0, 0, 0, 0, NULL)
     assert call(Hq=3) == _cabi.SAGE_EINVAL          # heads not divisible
     assert call(D=32) == _cabi.SAGE_ENOTIMPL
-    assert call(blkk=16) == _cabi.SAGE_ENOTIMPL      # attention needs scale blocks that are multiples of 32
+    assert call(blkk=8) == _cabi.SAGE_ENOTIMPL       # K scale blocks: 16, 32, 64 or 128 rows
+    assert call(blkq=16) == _cabi.SAGE_ENOTIMPL      # Q scale blocks: 32, 64 or 128 rows
     assert call(pv=1) == _cabi.SAGE_EINVAL           # fp8 needs v_scale
     assert call(pv=5) == _cabi.SAGE_EINVAL
 

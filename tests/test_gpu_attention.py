@@ -216,3 +216,42 @@ def test_lse_is_empty_unless_requested():
     qi, qs, ki, ks = sa.per_block_int8(q, q)
     out, lse = sa.forward(qi, ki, q, qs, ks)
     assert lse.numel() == 0 and out.dtype == torch.float16
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("pv", ["fp16", "fp8"])
+@pytest.mark.parametrize("D", [64, 128])
+def test_k_scale_blocks_of_16_keys(causal, pv, D):
+    # K granularity of the external recipe (128, 16) (sage_attention_benchmark_compare.py:93): two K scales per
+    # 32-key MFMA tile.  K gets a strong per-16-row amplitude pattern so that a wrong scale index cannot hide.
+    g = torch.Generator().manual_seed(31 + D)
+    B, Hq, Hkv, Sq, Skv = 1, 4, 2, 333, 421
+    q = randn("HND", B, Hq, Sq, D, torch.float16, g)
+    k = randn("HND", B, Hkv, Skv, D, torch.float16, g)
+    amp = (1.0 + 7.0 * ((torch.arange(Skv) // 16) % 3)).to(torch.float16)
+    k = k * amp[None, None, :, None]
+    v = randn("HND", B, Hkv, Skv, D, torch.float16, g)
+    qi, qs, ki, ks = sa.per_block_int8(q.to(DEV), k.to(DEV), BLKQ=128, BLKK=16)
+    assert tuple(ks.shape) == (B, Hkv, (Skv + 15) // 16)
+    out, lse = sa.forward(qi, ki, v.to(DEV), qs, ks, BLKQ=128, BLKK=16, is_causal=causal, pv_mode=pv, return_lse=True)
+    ref, ref_lse = oa.sage_reference(qi.cpu(), ki.cpu(), v, qs.cpu(), ks.cpu(), "HND", 128, 16, is_causal=causal)
+    m = oa.metrics(out.cpu().float(), ref)
+    assert m["finite"]
+    if pv == "fp16":
+        # the amplified K makes logits of ~100 (base 2): the fp32 constant that removes the accumulator bias,
+        # 1.5*2^23 * scale ~ 1e4, then carries ~1e-3 of rounding, which is what the LSE bound below allows
+        assert m["rel_rmse"] < 2e-3 and (lse.cpu().double() - ref_lse).abs().max().item() < 5e-3
+    else:
+        assert m["cosine"] >= 0.999 and m["rel_rmse"] < 5e-2
+
+
+def test_sageattn_with_the_128_16_recipe_against_fp32_sdpa():
+    g = torch.Generator().manual_seed(32)
+    q = randn("NHD", 2, 8, 600, 128, torch.bfloat16, g)
+    k = randn("NHD", 2, 2, 600, 128, torch.bfloat16, g)
+    v = randn("NHD", 2, 2, 600, 128, torch.bfloat16, g)
+    out = sa.sageattn(q.to(DEV), k.to(DEV), v.to(DEV), tensor_layout="NHD", is_causal=True, BLKQ=128, BLKK=16, pv_mode="fp8")
+    ref = oa.sdpa_fp32(q, k, v, "NHD", True)
+    assert oa.metrics(out.cpu().float(), ref)["cosine"] >= 0.999
+    with pytest.raises(NotImplementedError):
+        sa.sageattn(q.to(DEV), k.to(DEV), v.to(DEV), tensor_layout="NHD", BLKQ=16, BLKK=16)

@@ -76,7 +76,7 @@ def test_forward_contract():
     with pytest.raises(ValueError):
         sa.forward(q, k, v, fake(1, 4, 2, dtype=torch.float32), ks)  # q_scale shape
     with pytest.raises(NotImplementedError):
-        sa.forward(q, k, v, qs, ks, BLKK=16)
+        sa.forward(q, k, v, qs, ks, BLKK=8)
     with pytest.raises(ValueError):
         sa.forward(q, k, v, qs, ks, tensor_layout="XYZ")
 
