@@ -186,6 +186,12 @@ int sage_varlen_plan(const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k, i
 }  // extern "C"
 
 namespace {
+struct QRawArg {   // fp16/bf16 Q to be quantised by the attention kernel itself (q / q_scale are then ignored)
+  const void* ptr = nullptr;
+  int dtype = 0;
+  float mult = 1.0f;
+};
+
 struct MaskArg {
   const void* ptr = nullptr;
   int kind = 0;
@@ -198,7 +204,7 @@ int attn_impl(const int8_t* q, const int8_t* k, const void* v_panels, const floa
               int64_t q_sh, int64_t q_sn, int64_t k_sb, int64_t k_sh, int64_t k_sn, int64_t o_sb, int64_t o_sh,
               int64_t o_sn, int blkq, int blkk, int is_causal, int pv_mode, int out_dtype, const int32_t* cu_seqlens_q,
               const int32_t* cu_seqlens_k, const int32_t* plan, int total_q, int64_t q_scale_sh, int64_t k_scale_sh,
-              int64_t panel_sh, const MaskArg& mask, const float* lse_offset, sage_stream_t stream) {
+              int64_t panel_sh, const MaskArg& mask, const float* lse_offset, const QRawArg& qraw, sage_stream_t stream) {
   if (int rc = check_common(B, Hq, Sq, D, out_dtype)) return rc;
   if (Hkv <= 0 || Hq % Hkv) return fail(SAGE_EINVAL, "query heads (%d) must be divisible by KV heads (%d)", Hq, Hkv);
   if (Skv < 0) return fail(SAGE_EINVAL, "negative kv length");
@@ -207,9 +213,11 @@ int attn_impl(const int8_t* q, const int8_t* k, const void* v_panels, const floa
     return fail(SAGE_ENOTIMPL, "attention needs Q scale blocks of 32/64/128 rows and K scale blocks of 16/32/64/128 rows (got %d/%d)", blkq, blkk);
   if (blkk == 16 && mask.ptr) return fail(SAGE_ENOTIMPL, "K scale blocks of 16 rows cannot be combined with an explicit mask");
   if (B == 0 || Hq == 0 || Sq == 0) return SAGE_OK;
-  if (!q || !k || !v_panels || !q_scale || !k_scale || !out) return fail(SAGE_EINVAL, "null tensor pointer");
+  if (!k || !v_panels || !k_scale || !out) return fail(SAGE_EINVAL, "null tensor pointer");
+  if (!qraw.ptr && (!q || !q_scale)) return fail(SAGE_EINVAL, "null tensor pointer");
+  if (qraw.ptr && (mask.ptr || blkk == 16)) return fail(SAGE_ENOTIMPL, "fused Q quantisation: not with a mask or K blocks of 16");
   if (pv_mode == SAGE_PV_FP8 && !v_scale) return fail(SAGE_EINVAL, "fp8 P.V needs v_scale");
-  if (int rc = check_stride16("q", q_sb, q_sh, q_sn, 1, q)) return rc;
+  if (int rc = check_stride16("q", q_sb, q_sh, q_sn, qraw.ptr ? 2 : 1, qraw.ptr ? qraw.ptr : q)) return rc;
   if (int rc = check_stride16("k", k_sb, k_sh, k_sn, 1, k)) return rc;
   if ((o_sb % 4) || (o_sh % 4) || (o_sn % 4) || reinterpret_cast<uintptr_t>(out) % 8)
     return fail(SAGE_EINVAL, "out: base pointer and strides must be 8-byte aligned");
@@ -235,6 +243,7 @@ int attn_impl(const int8_t* q, const int8_t* k, const void* v_panels, const floa
   a.nqt = (Sq + BM - 1) / BM;
   a.mask = mask.ptr; a.mask_kind = mask.kind; a.m_sb = mask.sb; a.m_sh = mask.sh; a.m_sm = mask.sm; a.m_sn = mask.sn;
   a.mask_mult = mask.mult; a.lse_offset = lse_offset;
+  a.q_raw = qraw.ptr; a.q_is_bf16 = qraw.dtype == SAGE_DT_BF16; a.q_mult = qraw.mult;
   int64_t grid;
   if (packed) {
     SagePlanLayout L = plan_layout(B, total_q);
@@ -261,7 +270,7 @@ int sage_attn_fwd(const int8_t* q, const int8_t* k, const void* v_panels, const 
                   int64_t o_sn, int blkq, int blkk, int is_causal, int pv_mode, int out_dtype, const int32_t* cu_seqlens_q,
                   const int32_t* cu_seqlens_k, const int32_t* plan, int total_q, int64_t q_scale_sh, int64_t k_scale_sh,
                   int64_t panel_sh, sage_stream_t stream) {
-  return attn_impl(q, k, v_panels, q_scale, k_scale, v_scale, out, lse, B, Hq, Hkv, Sq, Skv, D, q_sb, q_sh, q_sn, k_sb, k_sh, k_sn, o_sb, o_sh, o_sn, blkq, blkk, is_causal, pv_mode, out_dtype, cu_seqlens_q, cu_seqlens_k, plan, total_q, q_scale_sh, k_scale_sh, panel_sh, MaskArg(), nullptr, stream);
+  return attn_impl(q, k, v_panels, q_scale, k_scale, v_scale, out, lse, B, Hq, Hkv, Sq, Skv, D, q_sb, q_sh, q_sn, k_sb, k_sh, k_sn, o_sb, o_sh, o_sn, blkq, blkk, is_causal, pv_mode, out_dtype, cu_seqlens_q, cu_seqlens_k, plan, total_q, q_scale_sh, k_scale_sh, panel_sh, MaskArg(), nullptr, QRawArg(), stream);
 }
 
 int sage_attn_fwd_masked(const int8_t* q, const int8_t* k, const void* v_panels, const float* q_scale, const float* k_scale,
@@ -274,7 +283,7 @@ int sage_attn_fwd_masked(const int8_t* q, const int8_t* k, const void* v_panels,
   m.ptr = attn_mask; m.kind = mask_kind; m.sb = m_sb; m.sh = m_sh; m.sm = m_sm; m.sn = m_sn;
   return attn_impl(q, k, v_panels, q_scale, k_scale, v_scale, out, lse, B, Hq, Hkv, Sq, Skv, D, q_sb, q_sh, q_sn, k_sb, k_sh,
                    k_sn, o_sb, o_sh, o_sn, blkq, blkk, 0, pv_mode, out_dtype, nullptr, nullptr, nullptr, 0, 0, 0, 0, m, nullptr,
-                   stream);
+                   QRawArg(), stream);
 }
 
 // ---- one-call pipeline --------------------------------------------------------------------
@@ -387,13 +396,20 @@ int sage_sageattn_masked(const void* q, const void* k, const void* v, void* out,
     lse_off = (float*)(ws + w.lse_off);
     dot.vec = km; dot.out = lse_off; dot.sb = (int64_t)Hkv * D; dot.sh = D; dot.group = Hq / Hkv; dot.total = total_q;
   }
-  rc = quant_impl(q, q_i8, q_scale, nullptr, B, Hq, Sq, D, q_sb, q_sh, q_sn, q_sb, q_sh, q_sn, 0, 0, blkq,
-                  (float)((sm_scale > 0 ? sm_scale : 1.0 / sqrt((double)D)) * 1.44269504), dtype, cu_seqlens_q, cu_qblk, w.qs_sh,
-                  dot, stream);
-  if (rc) return rc;
+  // Q is quantised by the attention kernel itself (each q-tile exactly where it is consumed) unless a
+  // feature needs the standalone pass: an explicit mask, K blocks of 16, or the LSE correction.
+  const float q_mult = (float)((sm_scale > 0 ? sm_scale : 1.0 / sqrt((double)D)) * 1.44269504);
+  const bool fuse_q = !attn_mask && blkk != 16 && !lse_off;
+  if (!fuse_q) {
+    rc = quant_impl(q, q_i8, q_scale, nullptr, B, Hq, Sq, D, q_sb, q_sh, q_sn, q_sb, q_sh, q_sn, 0, 0, blkq, q_mult, dtype,
+                    cu_seqlens_q, cu_qblk, w.qs_sh, dot, stream);
+    if (rc) return rc;
+  }
   rc = sage_prep_v(v, panels, v_scale, stat, stat_bytes, B, Hkv, Skv, D, v_sb, v_sh, v_sn, dtype, pv_mode, cu_seqlens_k,
                    cu_panel, w.panel_sh, stream);
   if (rc) return rc;
+  QRawArg qr;
+  if (fuse_q) { qr.ptr = q; qr.dtype = dtype; qr.mult = q_mult; }
   MaskArg m;
   if (attn_mask) {
     // sageattn's additive mask is in natural-log units on top of sm_scale * q.k (test_sage_attention_mate.py:171-176)
@@ -401,7 +417,7 @@ int sage_sageattn_masked(const void* q, const void* k, const void* v, void* out,
   }
   return attn_impl(q_i8, k_i8, panels, q_scale, k_scale, pv_mode == SAGE_PV_FP8 ? v_scale : nullptr, out, lse, B, Hq, Hkv, Sq,
                    Skv, D, q_sb, q_sh, q_sn, k_sb, k_sh, k_sn, o_sb, o_sh, o_sn, blkq, blkk, is_causal, pv_mode, dtype,
-                   cu_seqlens_q, cu_seqlens_k, plan, total_q, w.qs_sh, w.ks_sh, w.panel_sh, m, lse_off, stream);
+                   cu_seqlens_q, cu_seqlens_k, plan, total_q, w.qs_sh, w.ks_sh, w.panel_sh, m, lse_off, qr, stream);
 }
 
 }  // extern "C"

@@ -89,7 +89,8 @@ __device__ inline int kswz(int n) {
 // MASK: 0 none, 1 boolean keep-mask (bytes), 2 additive fp32 bias in base-2 score units
 // (sageattention_triton.py:92-105), both [B, Hq, Sq, Skv] with element strides.
 // KSUB: K scale blocks per 32 keys (1 for blocks of 32/64/128 keys, 2 for blocks of 16 keys).
-template <int D, int NW, int BN, int PV, bool CAUSAL, bool MSUM, int MASK, int KSUB = 1>
+// QF: the kernel reads fp16/bf16 Q and quantises its own tile (same arithmetic as quant_int8_kernel).
+template <int D, int NW, int BN, int PV, bool CAUSAL, bool MSUM, int MASK, int KSUB = 1, bool QF = false>
 __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
   constexpr int GSH = SAGE_GSH;   // which bit of the wavefront index picks the group
   constexpr int BM = NW * 32;
@@ -167,12 +168,59 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
 
   // ---- Q operand: lane (m, h) holds bytes 32*ks + 16*h .. +15 of its row for every ks ----
   v4i qreg[KS];
-  {
+  float qscale;
+  if constexpr (!QF) {
     const int8_t* qp = a.q + qoff + (int64_t)min(my_row, Lq - 1) * a.q_sn + 16 * h;
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) qreg[ks] = *reinterpret_cast<const v4i*>(qp + 32 * ks);
+    qscale = qsp[min(row0, Lq - 1) >> a.blkq_shift];
+  } else {
+    // Quantise this wavefront's 32 rows here, exactly as quant_int8_kernel would
+    // (quant_per_block.py:38-46): x32 = fp32(x) * mult, scale = max|x32| / 127 over the scale block
+    // (32, 64 or 128 rows = 1, 2 or 4 wavefronts), q = trunc(x32 / scale + 0.5 sgn).  Rows past the
+    // end repeat the last row, which belongs to the same (last) scale block or to none.
+#pragma clang fp contract(off)
+    __shared__ float q_block_amax[NW];
+    const u16* qp = reinterpret_cast<const u16*>(a.q_raw) + qoff + (int64_t)min(my_row, Lq - 1) * a.q_sn + 16 * h;
+    float x[KS][16];
+    float amax = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+      const uint4* src = reinterpret_cast<const uint4*>(qp + 32 * ks);
+      uint4 raw[2] = {src[0], src[1]};
+      const u16* e = reinterpret_cast<const u16*>(raw);
+#pragma unroll
+      for (int i = 0; i < 16; i++) {
+        x[ks][i] = (a.q_is_bf16 ? bf16_to_f32(e[i]) : f16_to_f32(e[i])) * a.q_mult;
+        amax = fmaxf(amax, fabsf(x[ks][i]));
+      }
+    }
+    amax = wave_max(amax);
+    const int wpb = a.blkq >> 5;   // wavefronts per scale block
+    if (wpb > 1) {
+      if (lane == 0) q_block_amax[w] = amax;
+      __syncthreads();
+      const int w0 = w & ~(wpb - 1);
+      for (int i = 0; i < wpb; i++) amax = fmaxf(amax, q_block_amax[w0 + i]);
+    }
+    const float scale = fmaxf(amax / 127.0f, kScaleFloor);
+    const float rcp = 1.0f / scale;
+    const uint32_t sbits = __builtin_bit_cast(uint32_t, scale);
+    const bool fast = ((sbits & 0x7fffffu) != 0x7fffffu) && scale < 1.0e30f;
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+      uint32_t packed[4] = {0, 0, 0, 0};
+#pragma unroll
+      for (int i = 0; i < 16; i++) {
+        float z = fast ? div_by_uniform(x[ks][i], scale, rcp) : x[ks][i] / scale;
+        z = z + __builtin_copysignf(0.5f, z);
+        int qv = (int)z;
+        packed[i >> 2] |= (uint32_t)(qv & 0xff) << (8 * (i & 3));
+      }
+      qreg[ks] = v4i{(int)packed[0], (int)packed[1], (int)packed[2], (int)packed[3]};
+    }
+    qscale = scale;
   }
-  const float qscale = qsp[min(row0, Lq - 1) >> a.blkq_shift];
 
   v16i bias;
 #pragma unroll
@@ -542,11 +590,11 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
 }
 
 
-template <int D, int NW, int BN, int PV, bool CAUSAL, bool MSUM, int MASK, int KSUB = 1>
+template <int D, int NW, int BN, int PV, bool CAUSAL, bool MSUM, int MASK, int KSUB = 1, bool QF = false>
 static hipError_t launch_one(const AttnArgs& a, int grid, hipStream_t st) {
   constexpr int VESZ = PV ? 1 : 2;
   constexpr int smem = 2 * (BN * D + BN * D * VESZ);   // two K slots + two V slots
-  auto kern = attn_kernel<D, NW, BN, PV, CAUSAL, MSUM, MASK, KSUB>;
+  auto kern = attn_kernel<D, NW, BN, PV, CAUSAL, MSUM, MASK, KSUB, QF>;
   static bool attr_done = false;
   if (!attr_done) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem);

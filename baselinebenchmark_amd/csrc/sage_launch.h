@@ -77,6 +77,10 @@ struct AttnArgs {
   int64_t m_sb, m_sh, m_sm, m_sn;
   float mask_mult;          // additive masks are scaled by this before they are added
   const float* lse_offset;  // added to LSE2 per query row (same layout as lse) or null
+  // fused Q quantisation: fp16/bf16 Q with the strides of q (q and qs are then unused)
+  const void* q_raw;
+  int q_is_bf16;
+  float q_mult;
 };
 
 struct AttnConfig { int nw, bn; };
@@ -90,6 +94,7 @@ hipError_t launch_prep_v(const PrepVArgs& a, int dtype, int pv, int max_panels, 
 AttnConfig attn_config(int D, int pv, bool packed);
 hipError_t launch_attn(const AttnArgs& a, int D, int pv, bool causal, int grid, hipStream_t st);
 hipError_t launch_attn_masked(const AttnArgs& a, int D, int pv, int grid, hipStream_t st);
+hipError_t launch_attn_qfused(const AttnArgs& a, int D, int pv, bool causal, int grid, hipStream_t st);
 hipError_t launch_attn_k16(const AttnArgs& a, int D, int pv, bool causal, int grid, hipStream_t st);
 hipError_t launch_varlen_plan(const int32_t* cu_q, const int32_t* cu_k, int nseq, int total_q, int blkq, int blkk, int bm,
                               int bn, int causal, int32_t* plan, hipStream_t st);

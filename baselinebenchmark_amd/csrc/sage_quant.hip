@@ -14,19 +14,6 @@
 
 namespace sage {
 
-constexpr float kScaleFloor = 1.0e-12f;
-
-
-// Correctly rounded x / s for a wavefront-uniform divisor whose reciprocal r = RN(1/s) is given.
-// q0 = RN(x*r) is within 1 ulp of x/s; e = x - q0*s is exact in one FMA; RN(q0 + e*r) is then
-// the correctly rounded quotient (Markstein's correction step), provided s's significand is not
-// all ones and nothing under/overflows; the caller falls back to a true division otherwise.
-__device__ inline float div_by_uniform(float x, float s, float r) {
-  float q0 = x * r;
-  float e = __builtin_fmaf(-q0, s, x);
-  return __builtin_fmaf(e, r, q0);
-}
-
 // One workgroup (256 lanes) quantises one [blk, D] tile held entirely in registers:
 // pass 1 converts and reduces |x| to the tile maximum, pass 2 divides and rounds.
 // A lane owns 16 consecutive channels of a row (two 128-bit loads, one 128-bit store).

@@ -255,3 +255,25 @@ def test_sageattn_with_the_128_16_recipe_against_fp32_sdpa():
     assert oa.metrics(out.cpu().float(), ref)["cosine"] >= 0.999
     with pytest.raises(NotImplementedError):
         sa.sageattn(q.to(DEV), k.to(DEV), v.to(DEV), tensor_layout="NHD", BLKQ=16, BLKK=16)
+
+
+@pytest.mark.parametrize("layout", ["HND", "NHD"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("cfg", [(128, 64, "fp16", False, 64), (64, 128, "fp8", True, 128), (32, 32, "fp8", False, 128),
+                                 (128, 128, "fp16", True, 128)])
+def test_q_quantised_inside_the_attention_kernel_is_bit_identical_to_the_standalone_quantiser(layout, dtype, cfg):
+    # sageattn quantises each q-tile in the attention prologue; forward() consumes the output of the standalone
+    # quantiser.  Same K mean, same K/V preparation: the two results must agree bit for bit, tails included.
+    blkq, blkk, pv, causal, D = cfg
+    g = torch.Generator().manual_seed(41 + blkq + D)
+    B, Hq, Hkv, S = 2, 4, 2, 777
+    q = (randn(layout, B, Hq, S, D, dtype, g).float() * 3.0).to(dtype)
+    k = randn(layout, B, Hkv, S, D, dtype, g)
+    v = randn(layout, B, Hkv, S, D, dtype, g)
+    qd, kd, vd = q.to(DEV), k.to(DEV), v.to(DEV)
+    fused = sa.sageattn(qd, kd, vd, tensor_layout=layout, is_causal=causal, sm_scale=0.11, pv_mode=pv, BLKQ=blkq, BLKK=blkk)
+    km = sa.k_mean(kd, layout)
+    qi, qs, ki, ks = sa.per_block_int8(qd, kd, km=km, BLKQ=blkq, BLKK=blkk, sm_scale=0.11, tensor_layout=layout)
+    two_step, _ = sa.forward(qi, ki, vd, qs, ks, tensor_layout=layout, output_dtype=dtype, BLKQ=blkq, BLKK=blkk,
+                             is_causal=causal, pv_mode=pv)
+    assert torch.equal(fused, two_step)
