@@ -36,6 +36,8 @@ SIGNATURES = {
     "sage_varlen_plan": (c_int, [_P, _P, _I, _I, _I, _I, _I, _P, c_size_t, _P]),
     "sage_attn_fwd": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I,
                               _L, _L, _L, _L, _L, _L, _L, _L, _L, _I, _I, _I, _I, _I, _P, _P, _P, _I, _L, _L, _L, _P]),
+    "sage_attn_fwd_qfused": (c_int, [_P, _I, c_double, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I,
+                                     _L, _L, _L, _L, _L, _L, _L, _L, _L, _I, _I, _I, _I, _I, _P, _P, _P, _I, _L, _L, _P]),
     "sage_attn_fwd_masked": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I,
                                      _L, _L, _L, _L, _L, _L, _L, _L, _L, _I, _I, _I, _I, _P, _I, _L, _L, _L, _L, _P]),
     "sage_sageattn_workspace_bytes": (c_size_t, [_I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I]),

@@ -273,6 +273,21 @@ int sage_attn_fwd(const int8_t* q, const int8_t* k, const void* v_panels, const 
   return attn_impl(q, k, v_panels, q_scale, k_scale, v_scale, out, lse, B, Hq, Hkv, Sq, Skv, D, q_sb, q_sh, q_sn, k_sb, k_sh, k_sn, o_sb, o_sh, o_sn, blkq, blkk, is_causal, pv_mode, out_dtype, cu_seqlens_q, cu_seqlens_k, plan, total_q, q_scale_sh, k_scale_sh, panel_sh, MaskArg(), nullptr, QRawArg(), stream);
 }
 
+int sage_attn_fwd_qfused(const void* q, int q_dtype, double sm_scale, const int8_t* k, const void* v_panels,
+                         const float* k_scale, const float* v_scale, void* out, float* lse, int B, int Hq, int Hkv, int Sq,
+                         int Skv, int D, int64_t q_sb, int64_t q_sh, int64_t q_sn, int64_t k_sb, int64_t k_sh, int64_t k_sn,
+                         int64_t o_sb, int64_t o_sh, int64_t o_sn, int blkq, int blkk, int is_causal, int pv_mode,
+                         int out_dtype, const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k, const int32_t* plan,
+                         int total_q, int64_t k_scale_sh, int64_t panel_sh, sage_stream_t stream) {
+  if (q_dtype != SAGE_DT_F16 && q_dtype != SAGE_DT_BF16) return fail(SAGE_ETYPE, "q dtype flag %d is not fp16(0)/bf16(1)", q_dtype);
+  if (!q) return fail(SAGE_EINVAL, "null tensor pointer");
+  QRawArg qr;
+  qr.ptr = q; qr.dtype = q_dtype; qr.mult = (float)((sm_scale > 0 ? sm_scale : 1.0 / sqrt((double)D)) * 1.44269504);
+  return attn_impl(nullptr, k, v_panels, nullptr, k_scale, v_scale, out, lse, B, Hq, Hkv, Sq, Skv, D, q_sb, q_sh, q_sn, k_sb,
+                   k_sh, k_sn, o_sb, o_sh, o_sn, blkq, blkk, is_causal, pv_mode, out_dtype, cu_seqlens_q, cu_seqlens_k, plan,
+                   total_q, 0, k_scale_sh, panel_sh, MaskArg(), nullptr, qr, stream);
+}
+
 int sage_attn_fwd_masked(const int8_t* q, const int8_t* k, const void* v_panels, const float* q_scale, const float* k_scale,
                          const float* v_scale, void* out, float* lse, int B, int Hq, int Hkv, int Sq, int Skv, int D,
                          int64_t q_sb, int64_t q_sh, int64_t q_sn, int64_t k_sb, int64_t k_sh, int64_t k_sn, int64_t o_sb,

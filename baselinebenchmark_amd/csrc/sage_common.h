@@ -72,12 +72,8 @@ __host__ __device__ inline SagePlanLayout plan_layout(int nseq, int total_q) {
 // dtype helpers (bf16 handled as raw bits: widening is a shift, narrowing is RNE).
 // ---------------------------------------------------------------------------------------------
 __device__ inline float bf16_to_f32(u16 v) { return __builtin_bit_cast(float, (uint32_t)v << 16); }
-__device__ inline u16 f32_to_bf16(float f) {
-  uint32_t u = __builtin_bit_cast(uint32_t, f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (u16)((u >> 16) | 0x40);  // quiet NaN
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (u16)(u >> 16);
-}
+// narrowing: gfx950 has a hardware round-to-nearest-even conversion (v_cvt_pk_bf16_f32)
+__device__ inline u16 f32_to_bf16(float f) { return __builtin_bit_cast(u16, (__bf16)f); }
 __device__ inline float f16_to_f32(u16 v) { return (float)__builtin_bit_cast(_Float16, v); }
 __device__ inline u16 f32_to_f16(float f) { return __builtin_bit_cast(u16, (_Float16)f); }
 

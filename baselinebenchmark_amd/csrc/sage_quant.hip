@@ -54,11 +54,10 @@ __global__ void __launch_bounds__(256) quant_int8_kernel(QuantArgs a) {
 #pragma unroll
     for (int i = 0; i < 16; i++) kmv[i] = to_f32<DT>(p[i]);
   }
-  auto value = [&](u16 bits, int i) {   // the fp32 value that is quantised
-    float x = to_f32<DT>(bits);
-    if (has_km) x = to_f32<DT>(from_f32<DT>(x - kmv[i]));
-    return x * a.mult;
-  };
+  // k - km is rounded to the input dtype (quant_per_block.py:53-54: the subtraction happens in torch, in
+  // the tensor's dtype) once, while loading; both passes then see the rounded difference.
+  auto smoothed = [&](u16 bits, int i) { return has_km ? from_f32<DT>(to_f32<DT>(bits) - kmv[i]) : bits; };
+  auto value = [&](u16 bits) { return to_f32<DT>(bits) * a.mult; };   // the fp32 value that is quantised
 
   // Optional side output: the dot product of every (scaled) row with a per-(batch, kv-head) vector.
   // The one-call pipeline uses it with the K mean to return the LSE of the unsmoothed logits.
@@ -83,12 +82,20 @@ __global__ void __launch_bounds__(256) quant_int8_kernel(QuantArgs a) {
       const uint4* src = reinterpret_cast<const uint4*>(a.x + xbase + (int64_t)(n0 + r) * a.x_sn + tc * 16);
       raw[p][0] = src[0];
       raw[p][1] = src[1];
+      if (has_km) {
+        const u16* e = reinterpret_cast<const u16*>(raw[p]);
+        uint32_t d[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) d[i] = (uint32_t)smoothed(e[2 * i], 2 * i) | ((uint32_t)smoothed(e[2 * i + 1], 2 * i + 1) << 16);
+        raw[p][0] = make_uint4(d[0], d[1], d[2], d[3]);
+        raw[p][1] = make_uint4(d[4], d[5], d[6], d[7]);
+      }
       const u16* e = reinterpret_cast<const u16*>(raw[p]);
 #pragma unroll
-      for (int i = 0; i < 16; i++) amax = fmaxf(amax, fabsf(value(e[i], i)));
+      for (int i = 0; i < 16; i++) amax = fmaxf(amax, fabsf(value(e[i])));
       if (has_dot) {
 #pragma unroll
-        for (int i = 0; i < 16; i++) dsum = __builtin_fmaf(value(e[i], i), dvv[i], dsum);
+        for (int i = 0; i < 16; i++) dsum = __builtin_fmaf(value(e[i]), dvv[i], dsum);
       }
     }
     if (has_dot) {   // uniform branch; the TPR lanes of a row are neighbours inside one wavefront
@@ -119,7 +126,7 @@ __global__ void __launch_bounds__(256) quant_int8_kernel(QuantArgs a) {
       uint32_t packed[4] = {0, 0, 0, 0};
 #pragma unroll
       for (int i = 0; i < 16; i++) {
-        const float x = value(e[i], i);
+        const float x = value(e[i]);
         float z;
         if (fast) {
           // For |x| so small that the residual of the correction step is subnormal the quotient is

@@ -266,6 +266,48 @@ def forward(q, k, v, q_scale, k_scale, tensor_layout="HND", attn_mask=None, outp
     return out, lse
 
 
+@torch.no_grad()
+def forward_fused_q(q, k, v, k_scale, tensor_layout="HND", sm_scale=None, output_dtype=None, return_lse=False,
+                    BLKQ=128, BLKK=64, is_causal=False, pv_mode="fp16"):
+    """forward() for a floating-point ``q`` and an already quantised ``k``: each q-tile is quantised inside the
+    attention kernel (bit-identical to per_block_int8 on q followed by forward()).  For callers that keep K
+    quantised across calls.  ``k``/``k_scale`` as returned by per_block_int8; returns (out, lse) like forward()."""
+    _check_float("q", q)
+    _check_float("v", v)
+    if not isinstance(k, torch.Tensor) or not k.is_cuda or k.dtype != torch.int8 or not k.is_contiguous():
+        raise TypeError("k must be contiguous GPU INT8")
+    if k_scale.dtype != torch.float32:
+        raise TypeError("k_scale must be FP32")
+    output_dtype = q.dtype if output_dtype is None else output_dtype
+    if output_dtype not in (torch.float16, torch.bfloat16):
+        raise NotImplementedError("output_dtype must be FP16 or BF16")
+    B, Hq, Sq, D, qsb, qsh, qsn = _layout(q, tensor_layout)
+    Bk, Hkv, Skv, Dk, ksb, ksh, ksn = _layout(k, tensor_layout)
+    Bv, Hv, Sv, Dv, _, _, _ = _layout(v, tensor_layout)
+    if Dk != D or Dv != D or Sv != Skv or Hv != Hkv or Bk != B or Bv != B:
+        raise ValueError("incompatible q/k/v shapes")
+    if Hq % Hkv:
+        raise ValueError("query heads must be divisible by KV heads")
+    if D not in (64, 128):
+        raise NotImplementedError("head_dim must be 64 or 128")
+    if BLKQ not in (32, 64, 128) or BLKK not in (32, 64, 128):
+        raise NotImplementedError("the fused-Q kernel needs scale blocks of 32, 64 or 128 rows")
+    if tuple(k_scale.shape) != (B, Hkv, (Skv + BLKK - 1) // BLKK):
+        raise ValueError(f"k_scale has shape {tuple(k_scale.shape)}, expected {(B, Hkv, (Skv + BLKK - 1) // BLKK)}")
+    pv = _pv(pv_mode)
+    panels, v_scale = prepare_v(v, tensor_layout, pv)
+    out = torch.empty(q.shape, device=q.device, dtype=output_dtype)
+    _, _, _, _, osb, osh, osn = _layout(out, tensor_layout)
+    lse = torch.empty((B, Hq, Sq), device=q.device, dtype=torch.float32) if return_lse else torch.empty(0, device=q.device)
+    check(lib().sage_attn_fwd_qfused(_ptr(q), _dt(q.dtype), float(D ** -0.5 if sm_scale is None else sm_scale), _ptr(k),
+                                     _ptr(panels), _ptr(k_scale.contiguous()), _ptr(v_scale), _ptr(out),
+                                     _ptr(lse if return_lse else None),
+                                     B, Hq, Hkv, Sq, Skv, D, qsb, qsh, qsn, ksb, ksh, ksn, osb, osh, osn,
+                                     BLKQ, BLKK, int(bool(is_causal)), pv, _dt(output_dtype), None, None, None, 0, 0, 0,
+                                     _stream(q)))
+    return out, lse
+
+
 # ------------------------------------------------------------------------------------------------
 # one-call API
 # ------------------------------------------------------------------------------------------------

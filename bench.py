@@ -43,8 +43,9 @@ def blended_peak(pv: str) -> float:
 
 
 def time_attention_kernel(sa, S, w, iters: int):
-    """Average duration of the fused attention kernel alone (operands pre-quantised), HIP events on the
-    launch stream.  Returns milliseconds per launch."""
+    """Average duration of the fused attention kernel alone, HIP events on the launch stream: the variant
+    the one-call pipeline runs (K and V pre-quantised, Q quantised in the kernel's prologue).  Returns
+    milliseconds per launch."""
     import ctypes
     from baselinebenchmark_amd._cabi import check, lib
     kw = w.kwargs
@@ -63,10 +64,11 @@ def time_attention_kernel(sa, S, w, iters: int):
     stream = torch.cuda.current_stream()
 
     def launch():
-        check(lib().sage_attn_fwd(S._ptr(qi), S._ptr(ki), S._ptr(panels), S._ptr(qs), S._ptr(ks), S._ptr(vs), S._ptr(out), None,
-                                  B, Hq, Hkv, Sq, Skv, D, qsb, qsh, qsn, ksb, ksh, ksn, osb, osh, osn,
-                                  kw["BLKQ"], kw["BLKK"], int(w.causal), pv, S._dt(q.dtype), None, None, None, 0, 0, 0, 0,
-                                  ctypes.c_void_p(stream.cuda_stream)))
+        check(lib().sage_attn_fwd_qfused(S._ptr(q), S._dt(q.dtype), float(D ** -0.5), S._ptr(ki), S._ptr(panels), S._ptr(ks),
+                                         S._ptr(vs), S._ptr(out), None,
+                                         B, Hq, Hkv, Sq, Skv, D, qsb, qsh, qsn, ksb, ksh, ksn, osb, osh, osn,
+                                         kw["BLKQ"], kw["BLKK"], int(w.causal), pv, S._dt(q.dtype), None, None, None, 0, 0, 0,
+                                         ctypes.c_void_p(stream.cuda_stream)))
     for _ in range(3):
         launch()
     stream.synchronize()

@@ -152,6 +152,29 @@ int sage_attn_fwd(const int8_t* q, const int8_t* k, const void* v_panels,
                   sage_stream_t stream);
 
 /*
+ * Attention on a floating-point Q and already quantised K / V: every workgroup quantises its own
+ * q-tile in the prologue with the arithmetic of sage_quant_int8 (quant_per_block.py:38-46, Q multiplier
+ * (float)(sm_scale * 1.44269504) of :87; sm_scale <= 0 selects head_dim^-0.5), so the result is bit-identical
+ * to sage_quant_int8 on q followed by sage_attn_fwd, without the HBM round trip of the INT8 copy of q.
+ * This is what sage_sageattn runs; it also fits callers that keep K and V quantised (a KV cache) and
+ * bring a fresh q.  q: fp16/bf16 (q_dtype) with element strides; everything else as in sage_attn_fwd.
+ * No counterpart in the reference (its quantiser is always a separate launch, sageattention_triton.py:140-164).
+ */
+int sage_attn_fwd_qfused(const void* q, int q_dtype, double sm_scale,
+                         const int8_t* k, const void* v_panels,
+                         const float* k_scale, const float* v_scale,
+                         void* out, float* lse,
+                         int B, int Hq, int Hkv, int Sq, int Skv, int D,
+                         int64_t q_sb, int64_t q_sh, int64_t q_sn,
+                         int64_t k_sb, int64_t k_sh, int64_t k_sn,
+                         int64_t o_sb, int64_t o_sh, int64_t o_sn,
+                         int blkq, int blkk, int is_causal, int pv_mode, int out_dtype,
+                         const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+                         const int32_t* plan, int total_q,
+                         int64_t k_scale_sh, int64_t panel_sh,
+                         sage_stream_t stream);
+
+/*
  * The same with an explicit mask: the attn_mask argument of forward
  * (sageattention_triton.py:167-168, :92-105; exercised by
  * backends/_hygon/test/sageattention/test_sageattention_hip.py:40-45, :65-66).

@@ -277,3 +277,19 @@ def test_q_quantised_inside_the_attention_kernel_is_bit_identical_to_the_standal
     two_step, _ = sa.forward(qi, ki, vd, qs, ks, tensor_layout=layout, output_dtype=dtype, BLKQ=blkq, BLKK=blkk,
                              is_causal=causal, pv_mode=pv)
     assert torch.equal(fused, two_step)
+
+
+def test_forward_fused_q_entry_point_matches_quantise_then_forward_bitwise():
+    g = torch.Generator().manual_seed(51)
+    B, Hq, Hkv, Sq, Skv, D = 1, 4, 4, 300, 500, 128
+    q = randn("HND", B, Hq, Sq, D, torch.bfloat16, g).to(DEV)
+    k = randn("HND", B, Hkv, Skv, D, torch.bfloat16, g).to(DEV)
+    v = randn("HND", B, Hkv, Skv, D, torch.bfloat16, g).to(DEV)
+    qi, qs, ki, ks = sa.per_block_int8(q, k, BLKQ=64, BLKK=128)
+    a, la = sa.forward(qi, ki, v, qs, ks, output_dtype=torch.bfloat16, BLKQ=64, BLKK=128, pv_mode="fp8", return_lse=True)
+    b, lb = sa.forward_fused_q(q, ki, v, ks, BLKQ=64, BLKK=128, pv_mode="fp8", return_lse=True)
+    assert torch.equal(a, b) and torch.equal(la, lb)
+    with pytest.raises(TypeError):
+        sa.forward_fused_q(qi, ki, v, ks)          # q must be floating point
+    with pytest.raises(NotImplementedError):
+        sa.forward_fused_q(q, ki, v, ks, BLKK=16)
