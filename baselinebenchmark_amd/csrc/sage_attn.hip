@@ -66,7 +66,7 @@ AttnConfig attn_config(int D, int pv, bool packed) {
   (void)D; (void)packed;
   AttnConfig c;
   c.nw = 8;
-  c.bn = pv ? 128 : 64;
+  c.bn = 128;
   return c;
 }
 
@@ -77,7 +77,7 @@ hipError_t launch_attn(const AttnArgs& a, int D, int pv, bool causal, int grid, 
   if (a.blkk == 16) return launch_attn_k16(a, D, pv, causal, grid, st);
   const bool msum = pv && a.lse == nullptr;   // row sums on the matrix pipe unless LSE is wanted
 #define SAGE_ATTN(DD, PVV, BNN, MS) (causal ? launch_one<DD, 8, BNN, PVV, true, MS, 0>(a, grid, st) : launch_one<DD, 8, BNN, PVV, false, MS, 0>(a, grid, st))
-  if (D == 128) return pv ? (msum ? SAGE_ATTN(128, 1, 128, true) : SAGE_ATTN(128, 1, 128, false)) : SAGE_ATTN(128, 0, 64, false);
+  if (D == 128) return pv ? (msum ? SAGE_ATTN(128, 1, 128, true) : SAGE_ATTN(128, 1, 128, false)) : SAGE_ATTN(128, 0, 128, false);
   return pv ? (msum ? SAGE_ATTN(64, 1, 128, true) : SAGE_ATTN(64, 1, 128, false)) : SAGE_ATTN(64, 0, 128, false);
 #undef SAGE_ATTN
 }

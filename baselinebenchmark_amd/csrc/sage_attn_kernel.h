@@ -301,7 +301,6 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
   float sc[NSC];
   auto sci = [](int nt, int r) { return KSUB == 2 ? 2 * nt + r / 8 : nt; };
   float mloc = kNegInf;
-  v8h ph[NT][2];      // fp16 mode
 
   // ---- S^T = K . Q^T (int8 -> int32 on the biased accumulators), then mask and row maximum ----
   auto qk = [&](int j) {
@@ -450,11 +449,16 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
           c[sub] = MASK ? PSHIFT - m_used : __builtin_fmaf(-kBiasF, sc[nt * KSUB + sub], PSHIFT - m_used);
           mul[sub] = MASK ? 1.0f : sc[nt * KSUB + sub];
         }
+        // fp16 probabilities are packed in place: registers 0-7 of each accumulator take the 16 halves
+        // (v_cvt_pk_f16_f32, round to nearest even) once the two scores they replace have been consumed.
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-          float p = __builtin_amdgcn_exp2f(__builtin_fmaf(as_f(acc[nt][r]), mul[KSUB == 2 ? r / 8 : 0], c[KSUB == 2 ? r / 8 : 0]));
-          lsum += p;
-          ph[nt][r >> 3][r & 7] = (_Float16)p;
+        for (int r = 0; r < 16; r += 2) {
+          v2f pp;
+          pp[0] = __builtin_amdgcn_exp2f(__builtin_fmaf(as_f(acc[nt][r]), mul[KSUB == 2 ? r / 8 : 0], c[KSUB == 2 ? r / 8 : 0]));
+          pp[1] = __builtin_amdgcn_exp2f(__builtin_fmaf(as_f(acc[nt][r + 1]), mul[KSUB == 2 ? r / 8 : 0], c[KSUB == 2 ? r / 8 : 0]));
+          lsum += pp[0];
+          lsum += pp[1];
+          acc[nt][r >> 1] = __builtin_bit_cast(int, __builtin_convertvector(pp, v2h));
         }
       }
     }
@@ -505,7 +509,9 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
       for (int i = 0; i < NV; i++) {
         const int k16 = i / DTN, dt = i % DTN;
         if (i + VPF < NV) vf[i + VPF] = vfrag(i + VPF);
-        o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[i], ph[k16 >> 1][k16 & 1], o[dt], 0, 0, 0);
+        const int nt = k16 >> 1, half = k16 & 1;
+        const v4i pw = {acc[nt][4 * half], acc[nt][4 * half + 1], acc[nt][4 * half + 2], acc[nt][4 * half + 3]};
+        o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[i], __builtin_bit_cast(v8h, pw), o[dt], 0, 0, 0);
       }
       __builtin_amdgcn_sched_group_barrier(0x100, VPF, 0);
 #pragma unroll

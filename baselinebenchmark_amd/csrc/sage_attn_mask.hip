@@ -9,14 +9,14 @@ namespace sage {
 
 hipError_t launch_attn_masked(const AttnArgs& a, int D, int pv, int grid, hipStream_t st) {
 #define SAGE_ATTN_M(DD, PVV, BNN) (a.mask_kind == 1 ? launch_one<DD, 8, BNN, PVV, false, false, 1>(a, grid, st) : launch_one<DD, 8, BNN, PVV, false, false, 2>(a, grid, st))
-  if (D == 128) return pv ? SAGE_ATTN_M(128, 1, 128) : SAGE_ATTN_M(128, 0, 64);
+  if (D == 128) return pv ? SAGE_ATTN_M(128, 1, 128) : SAGE_ATTN_M(128, 0, 128);
   return pv ? SAGE_ATTN_M(64, 1, 128) : SAGE_ATTN_M(64, 0, 128);
 #undef SAGE_ATTN_M
 }
 
 hipError_t launch_attn_k16(const AttnArgs& a, int D, int pv, bool causal, int grid, hipStream_t st) {
 #define SAGE_ATTN_K(DD, PVV, BNN) (causal ? launch_one<DD, 8, BNN, PVV, true, false, 0, 2>(a, grid, st) : launch_one<DD, 8, BNN, PVV, false, false, 0, 2>(a, grid, st))
-  if (D == 128) return pv ? SAGE_ATTN_K(128, 1, 128) : SAGE_ATTN_K(128, 0, 64);
+  if (D == 128) return pv ? SAGE_ATTN_K(128, 1, 128) : SAGE_ATTN_K(128, 0, 128);
   return pv ? SAGE_ATTN_K(64, 1, 128) : SAGE_ATTN_K(64, 0, 128);
 #undef SAGE_ATTN_K
 }
