@@ -93,6 +93,7 @@ __device__ inline int kswz(int n) {
 template <int D, int NW, int BN, int PV, bool CAUSAL, bool MSUM, int MASK, int KSUB = 1, bool QF = false>
 __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
   constexpr int GSH = SAGE_GSH;   // which bit of the wavefront index picks the group
+  static_assert(NW == (2 << GSH), "the two groups pair wavefront w with w + NW/2");
   constexpr int BM = NW * 32;
   constexpr int NTHR = NW * 64;
   constexpr int KS = D / 32;   // contraction steps of S^T
@@ -273,23 +274,26 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
 #pragma unroll
   for (int i = 0; i < VPIECES; i++) voffv[i] = (i * NW + w) * 1024 + lane * 16;
   const int ktile_bytes = BN * (int)a.k_sn;
-  auto load_k = [&](int j) {
-    uint8_t* dst = kslot(j);
+  // dw: load the pieces of wavefront w + dw instead of this wavefront's own.  dw is a multiple of 4, so
+  // the rows move by a multiple of 16 and keep their swizzle: only the uniform offset changes.
+  auto load_k = [&](int j, int dw) {
+    uint8_t* dst = kslot(j) + dw * 1024;
     if (j * BN + BN <= Lk) {
+      const int uo = j * ktile_bytes + dw * (64 / CPR) * (int)a.k_sn;
 #pragma unroll
-      for (int i = 0; i < KPIECES; i++) dma16(krsrc, koffv[i], j * ktile_bytes, dst + (i * NW + w) * 1024);
+      for (int i = 0; i < KPIECES; i++) dma16(krsrc, koffv[i], uo, dst + (i * NW + w) * 1024);
     } else {
 #pragma unroll
       for (int i = 0; i < KPIECES; i++) {
-        const int sl = (i * NW + w) * 64 + lane, n = sl / CPR, cc = (sl % CPR) ^ kswz<D>(n);
+        const int sl = (i * NW + w + dw) * 64 + lane, n = sl / CPR, cc = (sl % CPR) ^ kswz<D>(n);
         dma16(krsrc, min(j * BN + n, Lk - 1) * (int)a.k_sn + 16 * cc, 0, dst + (i * NW + w) * 1024);
       }
     }
   };
-  auto load_v = [&](int j) {
-    uint8_t* dst = vslot(j);
+  auto load_v = [&](int j, int dw) {
+    uint8_t* dst = vslot(j) + dw * 1024;
 #pragma unroll
-    for (int i = 0; i < VPIECES; i++) dma16(vrsrc, voffv[i], j * VBYTES, dst + (i * NW + w) * 1024);
+    for (int i = 0; i < VPIECES; i++) dma16(vrsrc, voffv[i], j * VBYTES + dw * 1024, dst + (i * NW + w) * 1024);
   };
 
   // State that crosses phases: the raw scores of the tile in flight, its row maximum and scales, and
@@ -538,18 +542,22 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
       if (j >= 1 && j - 1 < wnt) pv(j - 1);
       if (j < wnt) { qk(j); rowmax(j); }
     };
-    load_k(0);
+    load_k(0, 0);
     load_scales(0);
     auto even_barrier = [&](int j) {
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // my pieces of K(j) and V(j-1) have landed
       lds_barrier();                                     // ... and everyone's; phase 2j-1 is over
-      if (j + 1 < ntiles) load_k(j + 1);
-      if (j < ntiles) load_v(j);
     };
     if (grp == 0) {
+      // The even phase is as long as group 1's softmax, which must not start late: all tile loads of the
+      // period are issued here, by the group whose matrix phase has slack, after its P.V.
+      constexpr int PARTNER = 1 << GSH;
       for (int j = 0; j <= ntiles; j++) {
         even_barrier(j);
-        mfma_phase(j);
+        if (j >= 1 && j - 1 < wnt) pv(j - 1);
+        if (j + 1 < ntiles) { load_k(j + 1, 0); load_k(j + 1, PARTNER); }
+        if (j < ntiles) { load_v(j, 0); load_v(j, PARTNER); }
+        if (j < wnt) { qk(j); rowmax(j); }
         lds_barrier();
         if (j < wnt) softmax(j);
       }
