@@ -1,0 +1,167 @@
+// Micro-benchmarks of the gfx950 units the attention kernel is priced against: the two MFMA
+// instructions it uses (operands from registers, and fed from LDS the way the kernel feeds them), LDS
+// reads, and the vector instructions of the softmax.  They give the denominators MEASURED on the
+// box next to the datasheet ones.  No counterpart in the reference: a measurement aid.
+//
+// One workgroup per compute unit, 1, 2 or 4 wavefronts per SIMD; the caller times the launch (the
+// in-kernel clock s_memtime does not advance at wall-clock rate when wavefronts share a SIMD).
+#include "sage_common.h"
+#include "../../include/sage_mi355x.h"
+
+namespace sage {
+namespace {
+
+constexpr int kMbLdsInts = 16384;   // 64 KB
+
+enum : int { MB_MFMA_I8 = 0, MB_MFMA_F8 = 1, MB_LDS = 2, MB_MFMA_I8_LDS = 3, MB_MFMA_F8_LDS = 4,
+             MB_FMA = 5, MB_EXP = 6, MB_CVT_FP8 = 7, MB_SOFTMAX_MIX = 8, MB_KINDS = 9 };
+
+template <int KIND>
+__global__ void __launch_bounds__(1024) microbench_kernel(int* sink, int iters, int active_waves, float s, float c) {
+  __shared__ __attribute__((aligned(16))) int buf[kMbLdsInts];
+  for (int i = threadIdx.x; i < kMbLdsInts; i += blockDim.x) buf[i] = i * 7 + 1;
+  __syncthreads();
+  if ((int)(threadIdx.x >> 6) >= active_waves) return;
+  const int lane = threadIdx.x & 63;
+  int result = 0;
+  if constexpr (KIND == MB_MFMA_I8 || KIND == MB_MFMA_I8_LDS || KIND == MB_LDS) {
+    // per iteration: 16 fragments of 1 KB (lane-linear, conflict free) and/or 16 MFMAs on four accumulators
+    const v4i* p = reinterpret_cast<const v4i*>(buf) + lane;
+    v4i q = {lane, 1, 2, 3};
+    v16i acc[4] = {};
+    v4i sum = {0, 0, 0, 0};
+    constexpr int N = 16, PF = 4;
+    for (int it = 0; it < iters; it++) {
+      const v4i* pp = p + (it & 3) * 1024;
+      v4i f[N];
+      if (KIND != MB_MFMA_I8) {
+#pragma unroll
+        for (int i = 0; i < PF; i++) f[i] = pp[i * 64];
+      }
+#pragma unroll
+      for (int i = 0; i < N; i++) {
+        if (KIND != MB_MFMA_I8 && i + PF < N) f[i + PF] = pp[(i + PF) * 64];
+        __builtin_amdgcn_sched_barrier(0);
+        if (KIND == MB_MFMA_I8) acc[i & 3] = __builtin_amdgcn_mfma_i32_32x32x32_i8(q, q, acc[i & 3], 0, 0, 0);
+        if (KIND == MB_LDS) sum ^= f[i];
+        if (KIND == MB_MFMA_I8_LDS) acc[i & 3] = __builtin_amdgcn_mfma_i32_32x32x32_i8(f[i], q, acc[i & 3], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    result = sum[0] ^ sum[1] ^ sum[2] ^ sum[3];
+    for (int k = 0; k < 4; k++) result ^= acc[k][0];
+  } else if constexpr (KIND == MB_MFMA_F8 || KIND == MB_MFMA_F8_LDS) {
+    // per iteration: 8 MFMAs f8f6f4 32x32x64 (2 KB fragment each when fed from LDS)
+    const v4i* p = reinterpret_cast<const v4i*>(buf) + lane;
+    v8i q8 = {lane, 1, 2, 3, 4, 5, 6, 7};
+    v16f acc[4] = {};
+    constexpr int N = 8, PF = 3;
+    for (int it = 0; it < iters; it++) {
+      const v4i* pp = p + (it & 3) * 1024;
+      auto ld = [&](int i) {
+        v4i lo = pp[(2 * i) * 64], hi = pp[(2 * i + 1) * 64];
+        return v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      };
+      v8i f[N];
+      if (KIND == MB_MFMA_F8_LDS) {
+#pragma unroll
+        for (int i = 0; i < PF; i++) f[i] = ld(i);
+      }
+#pragma unroll
+      for (int i = 0; i < N; i++) {
+        if (KIND == MB_MFMA_F8_LDS && i + PF < N) f[i + PF] = ld(i + PF);
+        __builtin_amdgcn_sched_barrier(0);
+        if (KIND == MB_MFMA_F8) acc[i & 3] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(q8, q8, acc[i & 3], 0, 0, 0, 0, 0, 0);
+        else acc[i & 3] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f[i], q8, acc[i & 3], 0, 0, 0, 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    for (int k = 0; k < 4; k++) result ^= (int)acc[k][0];
+  } else {
+    // vector ALU: 32 independent values per lane; MB_SOFTMAX_MIX = per value one fma, one exp2, half a packed fp8 conversion
+    float x[32];
+    int pk[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (int i = 0; i < 32; i++) x[i] = lane * 1e-3f + i * 0.01f;
+    for (int it = 0; it < iters; it++) {
+      if constexpr (KIND == MB_FMA) {
+#pragma unroll
+        for (int i = 0; i < 32; i++) x[i] = __builtin_fmaf(x[i], s, c);
+      } else if constexpr (KIND == MB_EXP) {
+#pragma unroll
+        for (int i = 0; i < 32; i++) x[i] = __builtin_amdgcn_exp2f(x[i]);
+      } else {
+        float p[32];
+#pragma unroll
+        for (int i = 0; i < 32; i++) p[i] = KIND == MB_SOFTMAX_MIX ? __builtin_amdgcn_exp2f(__builtin_fmaf(x[i], s, c)) : x[i];
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+          int d0 = __builtin_amdgcn_cvt_pk_fp8_f32(p[4 * i], p[4 * i + 1], pk[i], false);
+          pk[i] = __builtin_amdgcn_cvt_pk_fp8_f32(p[4 * i + 2], p[4 * i + 3], d0, true);
+        }
+        // nothing of an iteration is loop invariant or dead
+#pragma unroll
+        for (int i = 0; i < 8; i++) asm volatile("" : "+v"(pk[i]));
+#pragma unroll
+        for (int i = 0; i < 32; i++) asm volatile("" : "+v"(x[i]));
+      }
+    }
+    float r = 0.f;
+    for (int i = 0; i < 32; i++) r += x[i];
+    for (int i = 0; i < 8; i++) result ^= pk[i];
+    result ^= (int)r;
+  }
+  sink[blockIdx.x * 1024 + threadIdx.x] = result;
+}
+
+template <int KIND>
+hipError_t launch_mb(int* sink, int grid, int waves, int iters, hipStream_t st) {
+  microbench_kernel<KIND><<<dim3(grid), dim3(waves * 64), 0, st>>>(sink, iters, waves, 0.999f, 0.001f);
+  return hipGetLastError();
+}
+
+}  // namespace
+}  // namespace sage
+
+extern "C" {
+
+// Units of work one wavefront does per iteration of benchmark `kind` (MFMA: multiply-add operations
+// counted as 2; LDS: bytes read; vector ALU: instructions), or 0 for an unknown kind.
+double sage_microbench_units(int kind) {
+  using namespace sage;
+  switch (kind) {
+    case MB_MFMA_I8: case MB_MFMA_I8_LDS: return 16.0 * 2 * 32 * 32 * 32;
+    case MB_MFMA_F8: case MB_MFMA_F8_LDS: return 8.0 * 2 * 32 * 32 * 64;
+    case MB_LDS: return 16.0 * 1024;
+    case MB_FMA: case MB_EXP: return 32.0;
+    case MB_CVT_FP8: return 16.0;
+    case MB_SOFTMAX_MIX: return 80.0;
+    default: return 0.0;
+  }
+}
+
+// Launches benchmark `kind` on `grid` workgroups of 4 * waves_per_simd wavefronts (waves_per_simd 1, 2 or 4), `iters`
+// iterations each.  `sink` receives one int per thread (grid * 1024 ints).  Returns 0 or a negative SAGE_E* code.
+int sage_microbench(int kind, int grid, int waves_per_simd, int iters, void* sink, size_t sink_bytes, sage_stream_t stream) {
+  using namespace sage;
+  if (kind < 0 || kind >= MB_KINDS || grid <= 0 || grid > 65535 || iters <= 0 || !sink) return SAGE_EINVAL;
+  if (waves_per_simd != 1 && waves_per_simd != 2 && waves_per_simd != 4) return SAGE_EINVAL;
+  if (sink_bytes < (size_t)grid * 1024 * sizeof(int)) return SAGE_EWORKSPACE;
+  int* out = (int*)sink;
+  const int waves = 4 * waves_per_simd;
+  hipStream_t st = (hipStream_t)stream;
+  hipError_t e = hipSuccess;
+  switch (kind) {
+    case MB_MFMA_I8: e = launch_mb<MB_MFMA_I8>(out, grid, waves, iters, st); break;
+    case MB_MFMA_F8: e = launch_mb<MB_MFMA_F8>(out, grid, waves, iters, st); break;
+    case MB_LDS: e = launch_mb<MB_LDS>(out, grid, waves, iters, st); break;
+    case MB_MFMA_I8_LDS: e = launch_mb<MB_MFMA_I8_LDS>(out, grid, waves, iters, st); break;
+    case MB_MFMA_F8_LDS: e = launch_mb<MB_MFMA_F8_LDS>(out, grid, waves, iters, st); break;
+    case MB_FMA: e = launch_mb<MB_FMA>(out, grid, waves, iters, st); break;
+    case MB_EXP: e = launch_mb<MB_EXP>(out, grid, waves, iters, st); break;
+    case MB_CVT_FP8: e = launch_mb<MB_CVT_FP8>(out, grid, waves, iters, st); break;
+    default: e = launch_mb<MB_SOFTMAX_MIX>(out, grid, waves, iters, st); break;
+  }
+  return e == hipSuccess ? SAGE_OK : SAGE_ELAUNCH;
+}
+
+}  // extern "C"

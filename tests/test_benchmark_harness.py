@@ -63,3 +63,19 @@ def test_tiny_run_gates_then_times_and_writes_a_result_file(tmp_path):
     for key in ("backend", "device", "operator", "framework_version", "driver_version", "commit", "cases", "tolerance"):
         assert key in doc
     assert doc["cases"][0]["shape"] == [1, 4, 256, 64] and doc["cases"][0]["warmup"] == 1
+
+
+@pytest.mark.gpu
+def test_hw_rate_microbenchmarks_run_and_are_plausible():
+    """The micro-benchmarks behind the measured roofline denominators: every kind runs through the C ABI and the two
+    MFMA instructions reach at least half of the datasheet rate from registers (they measure 80-95 % on the box)."""
+    from baselinebenchmark_amd.benchmarks import hw_rates
+    rows = hw_rates.run(iters_mfma=500, iters_valu=2000)
+    assert len(rows) == 3 * len(hw_rates.KINDS)
+    best = {}
+    for r in rows:
+        assert r["seconds"] > 0
+        if r["unit"] == "ops":
+            best[r["kind"]] = max(best.get(r["kind"], 0.0), r["chip_TOPS"])
+    assert best[0] > 2500 and best[1] > 2500, best
+    assert best[3] <= best[0] * 1.05 and best[4] <= best[1] * 1.05, best   # feeding from LDS never beats registers
