@@ -293,3 +293,36 @@ def test_forward_fused_q_entry_point_matches_quantise_then_forward_bitwise():
         sa.forward_fused_q(qi, ki, v, ks)          # q must be floating point
     with pytest.raises(NotImplementedError):
         sa.forward_fused_q(q, ki, v, ks, BLKK=16)
+
+
+def test_config2_full_size_properties():
+    """BASELINE config 2 at its full size (B2 H32 S16384 D128 bf16 causal, Q blk 64 / K blk 128, FP8 P.V) through
+    properties that need no O(T^2) reference on the host:
+      * heads are independent: permuting the heads of q, k and v permutes the output, bit for bit;
+      * causality: with K smoothing off, changing keys and values past a position (values only in sign, so that
+        the per-channel V scales, which span the whole sequence, stay the same) leaves every output row of the
+        earlier q-tiles bit-identical, while later rows do change;
+      * two calls give identical bits; everything is finite; row 0 of every head is v[0] of that head."""
+    from baselinebenchmark_amd import workloads
+    w = workloads.make("c2", device=DEV)
+    q, k, v = w.q, w.k, w.v
+    kw = dict(tensor_layout="HND", is_causal=True, pv_mode="fp8", BLKQ=64, BLKK=128)
+    out = sa.sageattn(q, k, v, **kw)
+    assert torch.isfinite(out.float()).all()
+    assert torch.equal(out, sa.sageattn(q, k, v, **kw))
+    assert torch.allclose(out[:, :, 0].float(), v[:, :, 0].float(), atol=0.08, rtol=0.08)
+    perm = torch.randperm(q.shape[1], generator=torch.Generator().manual_seed(5)).to(DEV)
+    out_p = sa.sageattn(q[:, perm].contiguous(), k[:, perm].contiguous(), v[:, perm].contiguous(), **kw)
+    assert torch.equal(out_p, out[:, perm])
+    del out_p
+    cut = 9000   # not a multiple of any block size
+    base = sa.sageattn(q, k, v, smooth_k=False, **kw)
+    k2, v2 = k.clone(), v.clone()
+    k2[:, :, cut:] += 1.0
+    v2[:, :, cut:] *= -1.0
+    pert = sa.sageattn(q, k2, v2, smooth_k=False, **kw)
+    # K is quantised in blocks of 128 rows, a q-tile has 256 rows: the q-tiles that end before the K block holding
+    # `cut` read identical INT8 keys and identical fp8 values
+    lim = (cut // 256) * 256
+    assert torch.equal(pert[:, :, :lim], base[:, :, :lim])
+    assert not torch.equal(pert[:, :, lim + 256:], base[:, :, lim + 256:])
