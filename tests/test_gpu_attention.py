@@ -326,3 +326,24 @@ def test_config2_full_size_properties():
     lim = (cut // 256) * 256
     assert torch.equal(pert[:, :, :lim], base[:, :, :lim])
     assert not torch.equal(pert[:, :, lim + 256:], base[:, :, lim + 256:])
+
+
+def test_config3_full_size_properties():
+    """BASELINE config 3 at its full size (B1 S32760 H24 D128 bf16 NHD, non-causal, FP8 P.V, x20 outlier channels,
+    tail tile of 120 rows): deterministic, finite, heads independent bit for bit, and the rows of the last
+    (partial) q-tile equal those of a stand-alone call that holds only these queries."""
+    from baselinebenchmark_amd import workloads
+    w = workloads.make("c3", device=DEV)
+    out = sa.sageattn(w.q, w.k, w.v, **w.kwargs)
+    assert torch.isfinite(out.float()).all()
+    assert torch.equal(out, sa.sageattn(w.q, w.k, w.v, **w.kwargs))
+    perm = torch.randperm(w.q.shape[2], generator=torch.Generator().manual_seed(6)).to(DEV)
+    out_p = sa.sageattn(w.q[:, :, perm].contiguous(), w.k[:, :, perm].contiguous(), w.v[:, :, perm].contiguous(), **w.kwargs)
+    assert torch.equal(out_p, out[:, :, perm])
+    del out_p
+    # non-causal: every query row is independent of the other queries, so the last 32760 - 127*256 = 248 rows alone
+    # (same Q scale blocks: 32512 is a multiple of the Q block) give the same bits
+    S = w.q.shape[1]
+    start = (S // 256) * 256
+    tail = sa.sageattn(w.q[:, start:].contiguous(), w.k, w.v, **w.kwargs)
+    assert torch.equal(tail, out[:, start:])

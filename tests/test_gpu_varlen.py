@@ -63,3 +63,24 @@ def test_plan_orders_tiles_by_decreasing_cost_and_covers_every_tile():
     cost = [(c + 63) // 64 for c in cost]
     assert cost == sorted(cost, reverse=True)
     assert p[offs[2]:offs[2] + 7].tolist() == np.concatenate([[0], np.cumsum([(L + 127) // 128 for L in lens])]).tolist()
+
+
+def test_config4_full_size_sequences_are_independent():
+    """BASELINE config 4 at its full size (16 packed sequences of 512..32768 rows, Hq32/Hkv8, D128 bf16 causal, FP8
+    P.V): the packed call reproduces, bit for bit, a stand-alone call on each of three of its sequences (shortest,
+    longest, and one in between), is deterministic and finite."""
+    from baselinebenchmark_amd import workloads
+    w = workloads.make("c4", device=DEV)
+    lens = w.extra["lens"]
+    cu = w.cu_seqlens
+    args = (w.q, w.k, w.v, cu, cu, w.max_seqlen, w.max_seqlen)
+    out = sa.sageattn_varlen(*args, **w.kwargs)
+    assert out.shape == w.q.shape and torch.isfinite(out.float()).all()
+    assert torch.equal(out, sa.sageattn_varlen(*args, **w.kwargs))
+    order = sorted(range(len(lens)), key=lambda i: lens[i])
+    cu_host = cu.cpu()
+    for i in (order[0], order[len(order) // 2], order[-1]):
+        sl = slice(int(cu_host[i]), int(cu_host[i + 1]))
+        alone = sa.sageattn(w.q[sl].unsqueeze(0).contiguous(), w.k[sl].unsqueeze(0).contiguous(), w.v[sl].unsqueeze(0).contiguous(),
+                            tensor_layout="NHD", **w.kwargs)
+        assert torch.equal(out[sl], alone[0]), (i, lens[i])
