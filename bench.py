@@ -110,7 +110,9 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=30,
+                    help="untimed steps before the timed ones; the first dozen steps after idle run up to 30 %% slower "
+                         "while the GPU clocks ramp, so the default covers that transient")
     ap.add_argument("--workload", default="c2", choices=["c0", "c1", "c2", "c3", "c4"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=20.0)
