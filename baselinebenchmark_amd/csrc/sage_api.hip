@@ -219,8 +219,10 @@ int attn_impl(const int8_t* q, const int8_t* k, const void* v_panels, const floa
   if (pv_mode == SAGE_PV_FP8 && !v_scale) return fail(SAGE_EINVAL, "fp8 P.V needs v_scale");
   if (int rc = check_stride16("q", q_sb, q_sh, q_sn, qraw.ptr ? 2 : 1, qraw.ptr ? qraw.ptr : q)) return rc;
   if (int rc = check_stride16("k", k_sb, k_sh, k_sn, 1, k)) return rc;
-  if ((o_sb % 4) || (o_sh % 4) || (o_sn % 4) || reinterpret_cast<uintptr_t>(out) % 8)
-    return fail(SAGE_EINVAL, "out: base pointer and strides must be 8-byte aligned");
+  if (int rc = check_stride16("out", o_sb, o_sh, o_sn, 2, out)) return rc;   // rows are stored 16 bytes per lane
+  // tile loads address a row of one (batch, head) slice with 32-bit byte offsets
+  if ((int64_t)Skv * k_sn >= 0x7fffffff || (qraw.ptr && (int64_t)Sq * q_sn * 2 >= 0x7fffffff))
+    return fail(SAGE_ENOTIMPL, "a (batch, head) slice of q or k spans 2 GiB or more");
   const bool packed = cu_seqlens_q != nullptr;
   if (mask.ptr) {
     if (mask.kind != SAGE_MASK_BOOL && mask.kind != SAGE_MASK_ADDITIVE) return fail(SAGE_EINVAL, "mask kind %d unknown", mask.kind);

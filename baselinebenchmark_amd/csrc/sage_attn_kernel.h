@@ -86,6 +86,22 @@ __device__ inline int kswz(int n) {
   return (n / RPB) % CPR;
 }
 
+// Dynamic LDS of a kernel variant: two K slots + two V slots; a kernel that quantises its own Q also
+// stages the raw q-tile behind K slot 0 (over K slot 1 and the V slots, which are idle until the main
+// loop); FP8 kernels keep the D per-channel V scales behind all of that.
+template <int D, int NW, int BN, int PV, bool QF>
+constexpr int attn_tile_lds_bytes() {
+  constexpr int tiles = 2 * (BN * D + BN * D * (PV ? 1 : 2));
+  constexpr int qstage = BN * D + NW * 32 * D * 2;
+  return (QF && qstage > tiles) ? qstage : tiles;
+}
+template <int D, int NW, int BN, int PV, bool QF>
+constexpr int attn_lds_bytes() { return attn_tile_lds_bytes<D, NW, BN, PV, QF>() + (PV ? D * 4 : 0); }
+
+#ifdef SAGE_TIMING
+static __device__ long long g_dbg[64];
+__device__ inline long long rt() { return __builtin_amdgcn_s_memrealtime(); }
+#endif
 // MASK: 0 none, 1 boolean keep-mask (bytes), 2 additive fp32 bias in base-2 score units
 // (sageattention_triton.py:92-105), both [B, Hq, Sq, Skv] with element strides.
 // KSUB: K scale blocks per 32 keys (1 for blocks of 32/64/128 keys, 2 for blocks of 16 keys).
@@ -108,6 +124,9 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
 
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
+#ifdef SAGE_TIMING
+  const long long T0 = rt();
+#endif
   const int tid = threadIdx.x, lane = tid & 63;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);  // wavefront index: uniform, keep it scalar
   const int m = lane & 31, h = lane >> 5;
@@ -167,87 +186,6 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
   const int wave_end = (row0 < Lq) ? (CAUSAL ? min(Lk, row0 + 32) : Lk) : 0;
   const int wave_ntiles = (wave_end + BN - 1) / BN;
 
-  // ---- Q operand: lane (m, h) holds bytes 32*ks + 16*h .. +15 of its row for every ks ----
-  v4i qreg[KS];
-  float qscale;
-  if constexpr (!QF) {
-    const int8_t* qp = a.q + qoff + (int64_t)min(my_row, Lq - 1) * a.q_sn + 16 * h;
-#pragma unroll
-    for (int ks = 0; ks < KS; ks++) qreg[ks] = *reinterpret_cast<const v4i*>(qp + 32 * ks);
-    qscale = qsp[min(row0, Lq - 1) >> a.blkq_shift];
-  } else {
-    // Quantise this wavefront's 32 rows here, exactly as quant_int8_kernel would
-    // (quant_per_block.py:38-46): x32 = fp32(x) * mult, scale = max|x32| / 127 over the scale block
-    // (32, 64 or 128 rows = 1, 2 or 4 wavefronts), q = trunc(x32 / scale + 0.5 sgn).  Rows past the
-    // end repeat the last row, which belongs to the same (last) scale block or to none.
-#pragma clang fp contract(off)
-    __shared__ float q_block_amax[NW];
-    const u16* qp = reinterpret_cast<const u16*>(a.q_raw) + qoff + (int64_t)min(my_row, Lq - 1) * a.q_sn + 16 * h;
-    float x[KS][16];
-    float amax = 0.f;
-#pragma unroll
-    for (int ks = 0; ks < KS; ks++) {
-      const uint4* src = reinterpret_cast<const uint4*>(qp + 32 * ks);
-      uint4 raw[2] = {src[0], src[1]};
-      const u16* e = reinterpret_cast<const u16*>(raw);
-#pragma unroll
-      for (int i = 0; i < 16; i++) {
-        x[ks][i] = (a.q_is_bf16 ? bf16_to_f32(e[i]) : f16_to_f32(e[i])) * a.q_mult;
-        amax = fmaxf(amax, fabsf(x[ks][i]));
-      }
-    }
-    amax = wave_max(amax);
-    const int wpb = a.blkq >> 5;   // wavefronts per scale block
-    if (wpb > 1) {
-      if (lane == 0) q_block_amax[w] = amax;
-      __syncthreads();
-      const int w0 = w & ~(wpb - 1);
-      for (int i = 0; i < wpb; i++) amax = fmaxf(amax, q_block_amax[w0 + i]);
-    }
-    const float scale = fmaxf(amax / 127.0f, kScaleFloor);
-    const float rcp = 1.0f / scale;
-    const uint32_t sbits = __builtin_bit_cast(uint32_t, scale);
-    const bool fast = ((sbits & 0x7fffffu) != 0x7fffffu) && scale < 1.0e30f;
-#pragma unroll
-    for (int ks = 0; ks < KS; ks++) {
-      uint32_t packed[4] = {0, 0, 0, 0};
-#pragma unroll
-      for (int i = 0; i < 16; i++) {
-        float z = fast ? div_by_uniform(x[ks][i], scale, rcp) : x[ks][i] / scale;
-        z = z + __builtin_copysignf(0.5f, z);
-        int qv = (int)z;
-        packed[i >> 2] |= (uint32_t)(qv & 0xff) << (8 * (i & 3));
-      }
-      qreg[ks] = v4i{(int)packed[0], (int)packed[1], (int)packed[2], (int)packed[3]};
-    }
-    qscale = scale;
-  }
-
-  v16i bias;
-#pragma unroll
-  for (int i = 0; i < 16; i++) bias[i] = kBiasBits;
-  asm volatile("" : "+v"(bias));  // keep it in registers: it is the C operand of every first MFMA
-
-  v16f o[DTN];
-#pragma unroll
-  for (int dt = 0; dt < DTN; dt++)
-#pragma unroll
-    for (int i = 0; i < 16; i++) o[dt][i] = 0.f;
-  float m_used = kMInit, lsum = 0.f;
-  // MSUM (FP8 mode when no LSE is requested): the row sums come out of the matrix pipe too.  A V^T operand of all ones (fp8 1.0 = 0x38)
-  // makes every row of one extra 32x32 output tile equal to sum_n P[n][m], i.e. the softmax
-  // denominator of query row m -- of the very fp8 values that multiply V.  That removes one VALU add
-  // per score (the VALU, not the MFMA pipe, is the busier unit of this kernel).  The sum of rounded
-  // values is the right denominator for O but costs LSE accuracy on rows with few keys, so kernels
-  // that return LSE keep the fp32 VALU sum.
-  v16f osum;
-#pragma unroll
-  for (int i = 0; i < 16; i++) osum[i] = 0.f;
-  v8i ones;
-#pragma unroll
-  for (int i = 0; i < 8; i++) ones[i] = 0x38383838;
-  asm volatile("" : "+v"(ones));
-
   // ---- tile loads: global memory -> LDS directly (no registers), 1 KB per wavefront instruction ----
   // Lane l of a wavefront writes LDS bytes [16*l, 16*l+16) of the 1 KB piece, so the K swizzle is
   // applied on the global side: the lane fetches the 16-byte chunk that belongs in its slot.
@@ -295,6 +233,127 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
 #pragma unroll
     for (int i = 0; i < VPIECES; i++) dma16(vrsrc, voffv[i], j * VBYTES + dw * 1024, dst + (i * NW + w) * 1024);
   };
+
+  // The first K tile is requested before anything else waits on memory, and the per-channel V scales
+  // of the epilogue come along (4 bytes per lane, D / 64 wavefronts).
+  if (ntiles > 0) load_k(0, 0);
+  float* vs_lds = reinterpret_cast<float*>(smem + attn_tile_lds_bytes<D, NW, BN, PV, QF>());
+  if constexpr (PV == 1) {
+    if (w < D / 64) {
+      const __amdgpu_buffer_rsrc_t vsrsrc =
+          __builtin_amdgcn_make_buffer_rsrc((void*)(a.vs + ((int64_t)b * a.Hkv + kvh) * D), 0, D * 4, 0x00020000);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(vsrsrc, (__attribute__((address_space(3))) void*)(vs_lds + 64 * w), 4, lane * 4, w * 256, 0, 0);
+    }
+  }
+
+#ifdef SAGE_TIMING
+  long long P1 = 0, P2 = 0;
+  { int tmp = nkblk + ntiles + wave_ntiles; asm volatile("" : "+v"(tmp)); }
+  P1 = rt();
+#endif
+  // ---- Q operand: lane (m, h) holds bytes 32*ks + 16*h .. +15 of its row for every ks ----
+  v4i qreg[KS];
+  float qscale;
+  if constexpr (!QF) {
+    const int8_t* qp = a.q + qoff + (int64_t)min(my_row, Lq - 1) * a.q_sn + 16 * h;
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) qreg[ks] = *reinterpret_cast<const v4i*>(qp + 32 * ks);
+    qscale = qsp[min(row0, Lq - 1) >> a.blkq_shift];
+  } else {
+    // Quantise this wavefront's 32 rows here, exactly as quant_int8_kernel would
+    // (quant_per_block.py:38-46): x32 = fp32(x) * mult, scale = max|x32| / 127 over the scale block
+    // (32, 64 or 128 rows = 1, 2 or 4 wavefronts), q = trunc(x32 / scale + 0.5 sgn).  Rows past the
+    // end repeat the last row, which belongs to the same (last) scale block or to none.
+#pragma clang fp contract(off)
+    __shared__ float q_block_amax[NW];
+    // The raw rows of this wavefront come in through LDS (1 KB per instruction, whole rows, into a region
+    // that no tile uses before the first barrier of the main loop) instead of 32-byte pieces of 32 rows
+    // per instruction.  16-byte units of a row are XOR-swizzled with the row index, on the global side as
+    // for K.  Only this wavefront reads its region, so its own vmcnt wait is all the ordering needed.
+    constexpr int QUPR = D * 2 / 16, QRPP = 64 / QUPR, QPIECES = 32 * D * 2 / 1024;
+    uint8_t* qstage = smem + KBYTES + w * (32 * D * 2);
+    {
+      const __amdgpu_buffer_rsrc_t qrsrc =
+          __builtin_amdgcn_make_buffer_rsrc((void*)(reinterpret_cast<const u16*>(a.q_raw) + qoff), 0, 0x7fffffff, 0x00020000);
+#pragma unroll
+      for (int i = 0; i < QPIECES; i++) {
+        const int r = i * QRPP + lane / QUPR;
+        const int u = (lane % QUPR) ^ (r & (QUPR - 1));
+        dma16(qrsrc, min(row0 + r, Lq - 1) * (int)a.q_sn * 2 + 16 * u, 0, qstage + i * 1024);
+      }
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+    float x[KS][16];
+    float amax = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+      uint4 raw[2];
+#pragma unroll
+      for (int e = 0; e < 2; e++)
+        raw[e] = *reinterpret_cast<const uint4*>(qstage + m * (D * 2) + 16 * ((4 * ks + 2 * h + e) ^ (m & (QUPR - 1))));
+      const u16* e = reinterpret_cast<const u16*>(raw);
+#pragma unroll
+      for (int i = 0; i < 16; i++) {
+        x[ks][i] = (a.q_is_bf16 ? bf16_to_f32(e[i]) : f16_to_f32(e[i])) * a.q_mult;
+        amax = fmaxf(amax, fabsf(x[ks][i]));
+      }
+    }
+    amax = wave_max(amax);
+#ifdef SAGE_TIMING
+    asm volatile("" : "+v"(amax));
+    P2 = rt();
+#endif
+    const int wpb = a.blkq >> 5;   // wavefronts per scale block
+    if (wpb > 1) {
+      if (lane == 0) q_block_amax[w] = amax;
+      __syncthreads();
+      const int w0 = w & ~(wpb - 1);
+      for (int i = 0; i < wpb; i++) amax = fmaxf(amax, q_block_amax[w0 + i]);
+    }
+    const float scale = fmaxf(amax / 127.0f, kScaleFloor);
+    const float rcp = 1.0f / scale;
+    const uint32_t sbits = __builtin_bit_cast(uint32_t, scale);
+    const bool fast = ((sbits & 0x7fffffu) != 0x7fffffu) && scale < 1.0e30f;
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+      uint32_t packed[4] = {0, 0, 0, 0};
+#pragma unroll
+      for (int i = 0; i < 16; i++) {
+        float z = fast ? div_by_uniform(x[ks][i], scale, rcp) : x[ks][i] / scale;
+        z = z + __builtin_copysignf(0.5f, z);
+        int qv = (int)z;
+        packed[i >> 2] |= (uint32_t)(qv & 0xff) << (8 * (i & 3));
+      }
+      qreg[ks] = v4i{(int)packed[0], (int)packed[1], (int)packed[2], (int)packed[3]};
+    }
+    qscale = scale;
+  }
+
+
+  v16i bias;
+#pragma unroll
+  for (int i = 0; i < 16; i++) bias[i] = kBiasBits;
+  asm volatile("" : "+v"(bias));  // keep it in registers: it is the C operand of every first MFMA
+
+  v16f o[DTN];
+#pragma unroll
+  for (int dt = 0; dt < DTN; dt++)
+#pragma unroll
+    for (int i = 0; i < 16; i++) o[dt][i] = 0.f;
+  float m_used = kMInit, lsum = 0.f;
+  // MSUM (FP8 mode when no LSE is requested): the row sums come out of the matrix pipe too.  A V^T operand of all ones (fp8 1.0 = 0x38)
+  // makes every row of one extra 32x32 output tile equal to sum_n P[n][m], i.e. the softmax
+  // denominator of query row m -- of the very fp8 values that multiply V.  That removes one VALU add
+  // per score (the VALU, not the MFMA pipe, is the busier unit of this kernel).  The sum of rounded
+  // values is the right denominator for O but costs LSE accuracy on rows with few keys, so kernels
+  // that return LSE keep the fp32 VALU sum.
+  v16f osum;
+#pragma unroll
+  for (int i = 0; i < 16; i++) osum[i] = 0.f;
+  v8i ones;
+#pragma unroll
+  for (int i = 0; i < 8; i++) ones[i] = 0x38383838;
+  asm volatile("" : "+v"(ones));
 
   // State that crosses phases: the raw scores of the tile in flight, its row maximum and scales, and
   // the probabilities packed as the B operand of the second MFMA.
@@ -535,6 +594,11 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
   //   phase 2j+1: group 0: softmax(j)              group 1: P.V(j-1), Q.K^T(j)
   // K tile j is read in phases 2j and 2j+1, V tile j in phases 2j+2 and 2j+3; both are loaded one
   // whole period before their first use, into the slot whose last reader finished a barrier ago.
+#ifdef SAGE_TIMING
+  asm volatile("" : "+v"(qreg[0]));
+  const long long T1 = rt();
+  long long TL = T1;
+#endif
   if (ntiles > 0) {
     const int grp = (w >> GSH) & 1;
     const int wnt = wave_ntiles;
@@ -542,11 +606,13 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
       if (j >= 1 && j - 1 < wnt) pv(j - 1);
       if (j < wnt) { qk(j); rowmax(j); }
     };
-    load_k(0, 0);
     load_scales(0);
     auto even_barrier = [&](int j) {
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // my pieces of K(j) and V(j-1) have landed
       lds_barrier();                                     // ... and everyone's; phase 2j-1 is over
+#ifdef SAGE_TIMING
+      if (j == 0) TL = rt();
+#endif
     };
     if (grp == 0) {
       // The even phase is as long as group 1's softmax, which must not start late: all tile loads of the
@@ -571,17 +637,34 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
     }
   }
 
+#ifdef SAGE_TIMING
+  const long long T2 = rt();
+#endif
   // ---- epilogue: O = O^T / l (* v_scale), LSE2 = m + log2(l) ----
   if constexpr (MSUM) lsum = osum[0];   // already the full row sum (the MFMA contracts over both lane halves)
   else lsum = xchg32_sum(lsum);
   const float inv = lsum > 0.f ? 1.0f / lsum : 0.f;
+#ifdef SAGE_TIMING
+  long long E2 = 0;
+#endif
   if (my_row < Lq) {
     if (a.lse && h == 0) {
       // lse_offset: what K smoothing removed from every logit of this row (q . k_mean, base-2 units)
       const float shift = a.lse_offset ? a.lse_offset[lseoff + my_row] : 0.f;
       a.lse[lseoff + my_row] = lsum > 0.f ? m_used + __builtin_amdgcn_logf(lsum) - PSHIFT + shift : kNegInf;
     }
-    const int64_t orow = ooff + (int64_t)my_row * a.o_sn;
+  }
+  // O^T (lane = row, registers = channels) goes to memory through LDS: written as stored, a wavefront
+  // instruction would touch 16 bytes of 32 different rows; read back row-wise, it stores whole rows
+  // (16 bytes per lane, 64 / UPR rows per instruction).  Each wavefront uses a private 32-row region
+  // of the tile buffers, which every wavefront has finished reading at the barrier.  16-byte units of
+  // a row are XOR-swizzled with the row index so that neither direction piles up on LDS banks.
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // (the V scales, when the main loop did not run)
+  lds_barrier();
+  {
+    constexpr int UPR = D / 8;        // 16-byte units per output row
+    constexpr int RPI = 64 / UPR;     // rows per store instruction
+    uint8_t* stage = smem + w * (32 * D * 2);
 #pragma unroll
     for (int dt = 0; dt < DTN; dt++) {
 #pragma unroll
@@ -591,23 +674,50 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
 #pragma unroll
         for (int i = 0; i < 4; i++) {
           f[i] = o[dt][4 * q4 + i] * inv;
-          if constexpr (PV == 1) f[i] *= a.vs[((int64_t)b * a.Hkv + kvh) * D + d + i];
+          if constexpr (PV == 1) f[i] *= vs_lds[d + i];
         }
         u16 hv[4];
 #pragma unroll
         for (int i = 0; i < 4; i++) hv[i] = a.out_bf16 ? f32_to_bf16(f[i]) : f32_to_f16(f[i]);
         uint2 pkd = make_uint2((uint32_t)hv[0] | ((uint32_t)hv[1] << 16), (uint32_t)hv[2] | ((uint32_t)hv[3] << 16));
-        *reinterpret_cast<uint2*>(reinterpret_cast<u16*>(a.out) + orow + d) = pkd;
+        const int u = 4 * dt + q4;    // 16-byte unit of the row; h picks its half
+        *reinterpret_cast<uint2*>(stage + m * (D * 2) + ((u ^ (m & (UPR - 1))) * 16) + 8 * h) = pkd;
       }
     }
+    const int k16 = lane % UPR, rsub = lane / UPR;
+#pragma unroll
+    for (int i = 0; i < 32 / RPI; i++) {
+      const int r = i * RPI + rsub;
+      const uint4 val = *reinterpret_cast<const uint4*>(stage + r * (D * 2) + ((k16 ^ (r & (UPR - 1))) * 16));
+      if (row0 + r < Lq)
+        *reinterpret_cast<uint4*>(reinterpret_cast<u16*>(a.out) + ooff + (int64_t)(row0 + r) * a.o_sn + k16 * 8) = val;
+    }
   }
+#ifdef SAGE_TIMING
+  E2 = rt();
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  const long long T3 = rt();
+  if (lane == 0) {
+    const int base = (w == 0 ? 0 : (w == NW - 1 ? 8 : 16));
+    atomicAdd((unsigned long long*)&g_dbg[base + 0], (unsigned long long)(T1 - T0));
+    atomicAdd((unsigned long long*)&g_dbg[base + 1], (unsigned long long)(T2 - T1));
+    atomicAdd((unsigned long long*)&g_dbg[base + 2], (unsigned long long)(T3 - T2));
+    atomicAdd((unsigned long long*)&g_dbg[base + 3], (unsigned long long)ntiles);
+    atomicAdd((unsigned long long*)&g_dbg[base + 4], 1ull);
+    atomicAdd((unsigned long long*)&g_dbg[base + 5], (unsigned long long)wave_ntiles);
+    atomicAdd((unsigned long long*)&g_dbg[base + 6], (unsigned long long)(P1 - T0));
+    atomicAdd((unsigned long long*)&g_dbg[base + 7], (unsigned long long)(P2 - P1));
+    atomicAdd((unsigned long long*)&g_dbg[32 + base + 0], (unsigned long long)(E2 - T2));
+    atomicAdd((unsigned long long*)&g_dbg[32 + base + 1], (unsigned long long)(TL - T1));
+  }
+#endif
 }
 
 
 template <int D, int NW, int BN, int PV, bool CAUSAL, bool MSUM, int MASK, int KSUB = 1, bool QF = false>
 static hipError_t launch_one(const AttnArgs& a, int grid, hipStream_t st) {
   constexpr int VESZ = PV ? 1 : 2;
-  constexpr int smem = 2 * (BN * D + BN * D * VESZ);   // two K slots + two V slots
+  constexpr int smem = attn_lds_bytes<D, NW, BN, PV, QF>();
   auto kern = attn_kernel<D, NW, BN, PV, CAUSAL, MSUM, MASK, KSUB, QF>;
   static bool attr_done = false;
   if (!attr_done) {

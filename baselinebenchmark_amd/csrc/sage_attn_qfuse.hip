@@ -14,3 +14,11 @@ hipError_t launch_attn_qfused(const AttnArgs& a, int D, int pv, bool causal, int
 }
 
 }  // namespace sage
+
+#ifdef SAGE_TIMING
+extern "C" void sage_debug_timing(long long* out) {
+  hipMemcpyFromSymbol(out, HIP_SYMBOL(sage::g_dbg), sizeof(long long) * 64);
+  long long z[64] = {0};
+  hipMemcpyToSymbol(HIP_SYMBOL(sage::g_dbg), z, sizeof(z));
+}
+#endif
