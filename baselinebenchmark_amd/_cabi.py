@@ -11,7 +11,10 @@ import ctypes
 from ctypes import c_char_p, c_double, c_float, c_int, c_int64, c_size_t, c_void_p
 from pathlib import Path
 
-LIB_PATH = Path(__file__).resolve().parent / "csrc" / "libsage_mi355x.so"
+import os
+
+# SAGE_MI355X_LIB selects another build of the same library (the timing build); there is still no fallback.
+LIB_PATH = Path(os.environ.get("SAGE_MI355X_LIB") or Path(__file__).resolve().parent / "csrc" / "libsage_mi355x.so")
 
 SAGE_OK, SAGE_EINVAL, SAGE_ETYPE, SAGE_ENOTIMPL, SAGE_ELAUNCH, SAGE_EWORKSPACE = 0, -1, -2, -3, -4, -5
 DT_F16, DT_BF16 = 0, 1

@@ -1,0 +1,73 @@
+"""Where a q-tile's time goes inside the fused attention kernel: the timing build of the library stamps eight
+points of every workgroup on the GPU's constant-rate counter (entry, tile decoded, raw Q arrived, Q operand ready,
+first barrier of the main loop, main loop done, stores issued, stores acknowledged) and sums the intervals.
+
+    python -m baselinebenchmark_amd.build --timing
+    SAGE_MI355X_LIB=baselinebenchmark_amd/csrc/libsage_mi355x_timing.so python -m baselinebenchmark_amd.benchmarks.tile_timing
+
+Prints, per shape, the average per workgroup in nanoseconds for the first, the last and the other wavefronts.  The
+timing build is slower than the shipped one (the stamps and their atomics); the intervals are what it is for.  No
+counterpart in the reference: a measurement aid.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+
+import torch
+
+import baselinebenchmark_amd as sa
+from baselinebenchmark_amd._cabi import LIB_PATH, lib
+
+INTERVALS = ["decode + first requests", "raw Q arrives", "Q maximum + quantise", "first loop barrier", "main loop",
+             "epilogue to last store", "store acknowledge"]
+TICK_NS = 10.0   # s_memrealtime runs at 100 MHz
+
+
+def _read():
+    fn = getattr(lib(), "sage_tile_timing", None)
+    if fn is None:
+        raise SystemExit(f"{LIB_PATH} is not a timing build: run `python -m baselinebenchmark_amd.build --timing` and set "
+                         "SAGE_MI355X_LIB to csrc/libsage_mi355x_timing.so")
+    buf = (ctypes.c_ulonglong * 32)()
+    if fn(buf) != 0:
+        raise RuntimeError("sage_tile_timing failed")
+    return list(buf)
+
+
+def measure(B, H, S, D, causal, dtype=torch.bfloat16, pv_mode="fp8", blkq=64, blkk=128, launches=5):
+    g = torch.Generator(device="cuda").manual_seed(0)
+    q, k, v = (torch.randn((B, H, S, D), dtype=dtype, device="cuda", generator=g) for _ in range(3))
+    _, _, ki, ks = sa.per_block_int8(q, k, BLKQ=blkq, BLKK=blkk)
+    call = lambda: sa.forward_fused_q(q, ki, v, ks, is_causal=causal, pv_mode=pv_mode, BLKQ=blkq, BLKK=blkk)
+    for _ in range(10):
+        call()
+    _read()
+    for _ in range(launches):
+        call()
+    d = _read()
+    rows = {}
+    for cls, name in enumerate(("first wavefront", "last wavefront", "other wavefronts")):
+        n = max(d[cls * 8 + 7], 1)
+        rows[name] = [d[cls * 8 + i] * TICK_NS / n for i in range(7)]
+    tiles = d[24] / max(d[7], 1)
+    return rows, tiles
+
+
+def main():
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--shapes", default="2x32x16384x128:1,2x32x16384x128:0,16x32x4096x128:1,64x32x1024x128:1",
+                    help="comma-separated BxHxSxD:causal")
+    args = ap.parse_args()
+    for spec in args.shapes.split(","):
+        dims, causal = spec.split(":")
+        B, H, S, D = (int(x) for x in dims.split("x"))
+        rows, tiles = measure(B, H, S, D, bool(int(causal)))
+        print(f"B{B} H{H} S{S} D{D} causal={bool(int(causal))}: {tiles:.1f} K tiles per workgroup", flush=True)
+        for name, vals in rows.items():
+            parts = ", ".join(f"{lbl} {v:.0f}" for lbl, v in zip(INTERVALS, vals))
+            print(f"  {name:17s} total {sum(vals):8.0f} ns | {parts} | main loop per tile {vals[4] / max(tiles, 1e-9):.0f}", flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -28,9 +28,12 @@ def _hipcc() -> str:
     return os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
 
-def _compile(src: str) -> Path:
-    obj = CSRC / (src.replace(".hip", ".o"))
-    cmd = [_hipcc(), *FLAGS, "-c", str(CSRC / src), "-o", str(obj)]
+TIMING_LIB = CSRC / "libsage_mi355x_timing.so"   # same library with in-kernel interval timers (a measurement aid)
+
+
+def _compile(src: str, timing: bool = False) -> Path:
+    obj = CSRC / (src.replace(".hip", ".timing.o" if timing else ".o"))
+    cmd = [_hipcc(), *FLAGS, *(["-DSAGE_TIMING=1"] if timing else []), "-c", str(CSRC / src), "-o", str(obj)]
     res = subprocess.run(cmd, capture_output=True, text=True)
     noise = "is not a recognized feature for this target"
     err = "\n".join(l for l in res.stderr.splitlines() if noise not in l)
@@ -41,17 +44,20 @@ def _compile(src: str) -> Path:
     return obj
 
 
-def build(verbose: bool = True) -> Path:
+def build(verbose: bool = True, timing: bool = False) -> Path:
+    """Builds the library; ``timing=True`` builds the instrumented twin (``-DSAGE_TIMING=1``) next to it instead,
+    for ``python -m baselinebenchmark_amd.benchmarks.tile_timing``."""
+    lib = TIMING_LIB if timing else LIB
     with ThreadPoolExecutor(max_workers=len(SOURCES)) as ex:
-        objs = list(ex.map(_compile, SOURCES))
-    cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", *map(str, objs), "-o", str(LIB)]
+        objs = list(ex.map(lambda src: _compile(src, timing), SOURCES))
+    cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", *map(str, objs), "-o", str(lib)]
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError(f"link failed:\n{res.stderr}")
     if verbose:
-        print(f"built {LIB} ({LIB.stat().st_size} bytes)")
-    return LIB
+        print(f"built {lib} ({lib.stat().st_size} bytes)")
+    return lib
 
 
 if __name__ == "__main__":
-    build()
+    build(timing="--timing" in sys.argv[1:])

@@ -86,21 +86,34 @@ __device__ inline int kswz(int n) {
   return (n / RPB) % CPR;
 }
 
-// Dynamic LDS of a kernel variant: two K slots + two V slots; a kernel that quantises its own Q also
-// stages the raw q-tile behind K slot 0 (over K slot 1 and the V slots, which are idle until the main
-// loop); FP8 kernels keep the D per-channel V scales behind all of that.
-template <int D, int NW, int BN, int PV, bool QF>
+// LDS slots per tile stream = how far ahead tiles are requested (slots - 1 periods before their first
+// use).  Two periods pay where every q-tile streams the whole sequence (non-causal, FP8 P.V: +4...7 %
+// measured from 1k to 16k keys); for causal and FP16 P.V kernels one period measured 1-3 % faster.
+template <int PV, bool CAUSAL>
+constexpr int attn_tile_slots() { return (PV == 1 && !CAUSAL) ? 3 : 2; }
+
+// Dynamic LDS of a kernel variant: the K slots and as many V slots; a kernel that quantises its own Q also
+// stages the raw q-tile behind the K slots that are requested in the prologue (over slots that are idle
+// until the main loop); FP8 kernels keep the D per-channel V scales behind all of that.
+template <int D, int NW, int BN, int PV, bool CAUSAL, bool QF>
 constexpr int attn_tile_lds_bytes() {
-  constexpr int tiles = 2 * (BN * D + BN * D * (PV ? 1 : 2));
-  constexpr int qstage = BN * D + NW * 32 * D * 2;
+  constexpr int slots = attn_tile_slots<PV, CAUSAL>();
+  constexpr int tiles = slots * (BN * D + BN * D * (PV ? 1 : 2));
+  constexpr int qstage = (slots - 1) * BN * D + NW * 32 * D * 2;
   return (QF && qstage > tiles) ? qstage : tiles;
 }
-template <int D, int NW, int BN, int PV, bool QF>
-constexpr int attn_lds_bytes() { return attn_tile_lds_bytes<D, NW, BN, PV, QF>() + (PV ? D * 4 : 0); }
+template <int D, int NW, int BN, int PV, bool CAUSAL, bool QF>
+constexpr int attn_lds_bytes() { return attn_tile_lds_bytes<D, NW, BN, PV, CAUSAL, QF>() + (PV ? D * 4 : 0); }
 
+// Timing build (-DSAGE_TIMING=1, not the shipped library): every wavefront stamps eight points of its
+// tile on the constant-rate 100 MHz counter and adds the seven intervals to per-class sums (class 0 =
+// first wavefront, 1 = last, 2 = the others): [class][0..6] intervals in ticks, [class][7] wavefronts,
+// [3][0] = tiles.  SAGE_T(k, x) pins stamp k after the computation of x.
 #ifdef SAGE_TIMING
-static __device__ long long g_dbg[64];
-__device__ inline long long rt() { return __builtin_amdgcn_s_memrealtime(); }
+static __device__ unsigned long long g_tile_timing[32];
+#define SAGE_T(k, x) do { asm volatile("" : "+v"(x)); sage_ts[k] = __builtin_amdgcn_s_memrealtime(); } while (0)
+#else
+#define SAGE_T(k, x) do { } while (0)
 #endif
 // MASK: 0 none, 1 boolean keep-mask (bytes), 2 additive fp32 bias in base-2 score units
 // (sageattention_triton.py:92-105), both [B, Hq, Sq, Skv] with element strides.
@@ -121,11 +134,13 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
   constexpr int PANEL_BYTES = kPanelRows * D * VESZ;
   constexpr int CPR = D / 16;
   constexpr float TAU = PCfg<PV>::tau, PSHIFT = PCfg<PV>::pshift;
+  constexpr int NSLOT = attn_tile_slots<PV, CAUSAL>(), LEAD = NSLOT - 1;   // tiles are requested LEAD periods ahead
 
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
 #ifdef SAGE_TIMING
-  const long long T0 = rt();
+  long long sage_ts[8];
+  for (int i = 0; i < 8; i++) sage_ts[i] = __builtin_amdgcn_s_memrealtime();
 #endif
   const int tid = threadIdx.x, lane = tid & 63;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);  // wavefront index: uniform, keep it scalar
@@ -189,7 +204,7 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
   // ---- tile loads: global memory -> LDS directly (no registers), 1 KB per wavefront instruction ----
   // Lane l of a wavefront writes LDS bytes [16*l, 16*l+16) of the 1 KB piece, so the K swizzle is
   // applied on the global side: the lane fetches the 16-byte chunk that belongs in its slot.
-  // K tiles and V tiles each alternate between two LDS slots.
+  // K tiles and V tiles each rotate through NSLOT LDS slots.
   constexpr int KPIECES = KBYTES / 1024 / NW, VPIECES = VBYTES / 1024 / NW;
   static_assert(KPIECES * 1024 * NW == KBYTES && VPIECES * 1024 * NW == VBYTES, "tile must split into 1 KB pieces per wavefront");
   // The buffer form of the LDS load is used on purpose: the compiler treats the global form as a flat
@@ -199,8 +214,8 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
   auto dma16 = [&](__amdgpu_buffer_rsrc_t rsrc, int lane_offset, int uniform_offset, uint8_t* dst_uniform) {
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)dst_uniform, 16, lane_offset, uniform_offset, 0, 0);
   };
-  auto kslot = [&](int j) { return smem + (j & 1) * KBYTES; };
-  auto vslot = [&](int j) { return smem + 2 * KBYTES + (j & 1) * VBYTES; };
+  auto kslot = [&](int j) { return smem + (j % NSLOT) * KBYTES; };
+  auto vslot = [&](int j) { return smem + NSLOT * KBYTES + (j % NSLOT) * VBYTES; };
   // Per-lane byte offsets of this wavefront's pieces inside a tile are loop invariant; the tile index
   // only adds a uniform term.  Rows past the end of the sequence (last tile only) are clamped.
   int koffv[KPIECES], voffv[VPIECES];
@@ -237,7 +252,7 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
   // The first K tile is requested before anything else waits on memory, and the per-channel V scales
   // of the epilogue come along (4 bytes per lane, D / 64 wavefronts).
   if (ntiles > 0) load_k(0, 0);
-  float* vs_lds = reinterpret_cast<float*>(smem + attn_tile_lds_bytes<D, NW, BN, PV, QF>());
+  float* vs_lds = reinterpret_cast<float*>(smem + attn_tile_lds_bytes<D, NW, BN, PV, CAUSAL, QF>());
   if constexpr (PV == 1) {
     if (w < D / 64) {
       const __amdgpu_buffer_rsrc_t vsrsrc =
@@ -246,11 +261,7 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
     }
   }
 
-#ifdef SAGE_TIMING
-  long long P1 = 0, P2 = 0;
-  { int tmp = nkblk + ntiles + wave_ntiles; asm volatile("" : "+v"(tmp)); }
-  P1 = rt();
-#endif
+  { [[maybe_unused]] int addressed = nkblk + ntiles + wave_ntiles; SAGE_T(1, addressed); }   // tile decoded, first loads requested
   // ---- Q operand: lane (m, h) holds bytes 32*ks + 16*h .. +15 of its row for every ks ----
   v4i qreg[KS];
   float qscale;
@@ -271,7 +282,7 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
     // per instruction.  16-byte units of a row are XOR-swizzled with the row index, on the global side as
     // for K.  Only this wavefront reads its region, so its own vmcnt wait is all the ordering needed.
     constexpr int QUPR = D * 2 / 16, QRPP = 64 / QUPR, QPIECES = 32 * D * 2 / 1024;
-    uint8_t* qstage = smem + KBYTES + w * (32 * D * 2);
+    uint8_t* qstage = smem + LEAD * KBYTES + w * (32 * D * 2);
     {
       const __amdgpu_buffer_rsrc_t qrsrc =
           __builtin_amdgcn_make_buffer_rsrc((void*)(reinterpret_cast<const u16*>(a.q_raw) + qoff), 0, 0x7fffffff, 0x00020000);
@@ -299,10 +310,7 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
       }
     }
     amax = wave_max(amax);
-#ifdef SAGE_TIMING
-    asm volatile("" : "+v"(amax));
-    P2 = rt();
-#endif
+    SAGE_T(2, amax);   // the raw Q rows have arrived
     const int wpb = a.blkq >> 5;   // wavefronts per scale block
     if (wpb > 1) {
       if (lane == 0) q_block_amax[w] = amax;
@@ -329,6 +337,9 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
     qscale = scale;
   }
 
+
+  // With two periods of lead the second K tile follows as soon as the raw Q rows are out of the way.
+  if (LEAD == 2 && ntiles > 1) load_k(1, 0);
 
   v16i bias;
 #pragma unroll
@@ -592,13 +603,8 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
   // are kept busy at the same time instead of taking turns.
   //   phase 2j  : group 0: P.V(j-1), Q.K^T(j)      group 1: softmax(j-1)
   //   phase 2j+1: group 0: softmax(j)              group 1: P.V(j-1), Q.K^T(j)
-  // K tile j is read in phases 2j and 2j+1, V tile j in phases 2j+2 and 2j+3; both are loaded one
-  // whole period before their first use, into the slot whose last reader finished a barrier ago.
-#ifdef SAGE_TIMING
-  asm volatile("" : "+v"(qreg[0]));
-  const long long T1 = rt();
-  long long TL = T1;
-#endif
+  // K tile j is read in phases 2j and 2j+1, V tile j in phases 2j+2 and 2j+3.
+  SAGE_T(3, qreg[0]);   // Q operand ready
   if (ntiles > 0) {
     const int grp = (w >> GSH) & 1;
     const int wnt = wave_ntiles;
@@ -607,29 +613,51 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
       if (j < wnt) { qk(j); rowmax(j); }
     };
     load_scales(0);
-    auto even_barrier = [&](int j) {
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // my pieces of K(j) and V(j-1) have landed
-      lds_barrier();                                     // ... and everyone's; phase 2j-1 is over
+    // Tile loads complete in the order they were requested, so waiting until only the n newest are in
+    // flight leaves exactly the requests of the last period outstanding.
+    auto wait_all_but = [&](int n) {
+      switch (n) {
+        case 0: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+        case 1: asm volatile("s_waitcnt vmcnt(1)" ::: "memory"); break;
+        case 2: asm volatile("s_waitcnt vmcnt(2)" ::: "memory"); break;
+        case 3: asm volatile("s_waitcnt vmcnt(3)" ::: "memory"); break;
+        case 4: asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); break;
+        case 6: asm volatile("s_waitcnt vmcnt(6)" ::: "memory"); break;
+        case 8: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
+        case 10: asm volatile("s_waitcnt vmcnt(10)" ::: "memory"); break;
+        case 12: asm volatile("s_waitcnt vmcnt(12)" ::: "memory"); break;
+        default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+      }
+    };
+    auto even_barrier = [&](int j, int in_flight) {
+      wait_all_but(in_flight);   // my pieces of K(j) and V(j-1) have landed
+      lds_barrier();             // ... and everyone's; phase 2j-1 is over
 #ifdef SAGE_TIMING
-      if (j == 0) TL = rt();
+      if (j == 0) sage_ts[4] = __builtin_amdgcn_s_memrealtime();   // first K tile landed, all wavefronts arrived
 #endif
     };
+    const int first_in_flight = (LEAD == 2 && ntiles > 1) ? KPIECES : 0;   // the second K tile, requested in the prologue
     if (grp == 0) {
       // The even phase is as long as group 1's softmax, which must not start late: all tile loads of the
-      // period are issued here, by the group whose matrix phase has slack, after its P.V.
+      // period are issued here, by the group whose matrix phase has slack, after its P.V.  Period j requests
+      // K(j+LEAD) and V(j+LEAD-1), LEAD periods before their first use (a tile that has to come from HBM takes
+      // longer than one period), into the slots whose last readers finished a barrier ago; with LEAD = 2,
+      // V(0) goes first in period 0 and the requests of the last period may still be in flight at a barrier.
       constexpr int PARTNER = 1 << GSH;
+      constexpr int NK = 2 * KPIECES, NV = 2 * VPIECES;   // requests per K / V tile of a group-0 wavefront
       for (int j = 0; j <= ntiles; j++) {
-        even_barrier(j);
+        even_barrier(j, j == 0 ? first_in_flight : LEAD == 1 ? 0 : (j + 1 < ntiles ? NK : 0) + (j < ntiles ? NV : 0));
         if (j >= 1 && j - 1 < wnt) pv(j - 1);
-        if (j + 1 < ntiles) { load_k(j + 1, 0); load_k(j + 1, PARTNER); }
-        if (j < ntiles) { load_v(j, 0); load_v(j, PARTNER); }
+        if (LEAD == 2 && j == 0) { load_v(0, 0); load_v(0, PARTNER); }
+        if (j + LEAD < ntiles) { load_k(j + LEAD, 0); load_k(j + LEAD, PARTNER); }
+        if (j + LEAD - 1 < ntiles) { load_v(j + LEAD - 1, 0); load_v(j + LEAD - 1, PARTNER); }
         if (j < wnt) { qk(j); rowmax(j); }
         lds_barrier();
         if (j < wnt) softmax(j);
       }
     } else {
       for (int j = 0; j <= ntiles; j++) {
-        even_barrier(j);
+        even_barrier(j, j == 0 ? first_in_flight : 0);
         if (j >= 1 && j - 1 < wnt) softmax(j - 1);
         lds_barrier();
         mfma_phase(j);
@@ -637,16 +665,11 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
     }
   }
 
-#ifdef SAGE_TIMING
-  const long long T2 = rt();
-#endif
+  SAGE_T(5, lsum);   // main loop done
   // ---- epilogue: O = O^T / l (* v_scale), LSE2 = m + log2(l) ----
   if constexpr (MSUM) lsum = osum[0];   // already the full row sum (the MFMA contracts over both lane halves)
   else lsum = xchg32_sum(lsum);
   const float inv = lsum > 0.f ? 1.0f / lsum : 0.f;
-#ifdef SAGE_TIMING
-  long long E2 = 0;
-#endif
   if (my_row < Lq) {
     if (a.lse && h == 0) {
       // lse_offset: what K smoothing removed from every logit of this row (q . k_mean, base-2 units)
@@ -694,21 +717,15 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
     }
   }
 #ifdef SAGE_TIMING
-  E2 = rt();
+  sage_ts[6] = __builtin_amdgcn_s_memrealtime();   // stores issued
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  const long long T3 = rt();
+  sage_ts[7] = __builtin_amdgcn_s_memrealtime();   // stores acknowledged
+  if (ntiles == 0) sage_ts[4] = sage_ts[3];
   if (lane == 0) {
-    const int base = (w == 0 ? 0 : (w == NW - 1 ? 8 : 16));
-    atomicAdd((unsigned long long*)&g_dbg[base + 0], (unsigned long long)(T1 - T0));
-    atomicAdd((unsigned long long*)&g_dbg[base + 1], (unsigned long long)(T2 - T1));
-    atomicAdd((unsigned long long*)&g_dbg[base + 2], (unsigned long long)(T3 - T2));
-    atomicAdd((unsigned long long*)&g_dbg[base + 3], (unsigned long long)ntiles);
-    atomicAdd((unsigned long long*)&g_dbg[base + 4], 1ull);
-    atomicAdd((unsigned long long*)&g_dbg[base + 5], (unsigned long long)wave_ntiles);
-    atomicAdd((unsigned long long*)&g_dbg[base + 6], (unsigned long long)(P1 - T0));
-    atomicAdd((unsigned long long*)&g_dbg[base + 7], (unsigned long long)(P2 - P1));
-    atomicAdd((unsigned long long*)&g_dbg[32 + base + 0], (unsigned long long)(E2 - T2));
-    atomicAdd((unsigned long long*)&g_dbg[32 + base + 1], (unsigned long long)(TL - T1));
+    const int cls = w == 0 ? 0 : (w == NW - 1 ? 1 : 2);
+    for (int i = 0; i < 7; i++) atomicAdd(&g_tile_timing[cls * 8 + i], (unsigned long long)(sage_ts[i + 1] - sage_ts[i]));
+    atomicAdd(&g_tile_timing[cls * 8 + 7], 1ull);
+    if (w == 0) atomicAdd(&g_tile_timing[24], (unsigned long long)ntiles);
   }
 #endif
 }
@@ -717,7 +734,7 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
 template <int D, int NW, int BN, int PV, bool CAUSAL, bool MSUM, int MASK, int KSUB = 1, bool QF = false>
 static hipError_t launch_one(const AttnArgs& a, int grid, hipStream_t st) {
   constexpr int VESZ = PV ? 1 : 2;
-  constexpr int smem = attn_lds_bytes<D, NW, BN, PV, QF>();
+  constexpr int smem = attn_lds_bytes<D, NW, BN, PV, CAUSAL, QF>();
   auto kern = attn_kernel<D, NW, BN, PV, CAUSAL, MSUM, MASK, KSUB, QF>;
   static bool attr_done = false;
   if (!attr_done) {

@@ -16,9 +16,12 @@ hipError_t launch_attn_qfused(const AttnArgs& a, int D, int pv, bool causal, int
 }  // namespace sage
 
 #ifdef SAGE_TIMING
-extern "C" void sage_debug_timing(long long* out) {
-  hipMemcpyFromSymbol(out, HIP_SYMBOL(sage::g_dbg), sizeof(long long) * 64);
-  long long z[64] = {0};
-  hipMemcpyToSymbol(HIP_SYMBOL(sage::g_dbg), z, sizeof(z));
+// Timing build only: copies the interval sums of the kernels of this translation unit (the ones the one-call
+// pipeline runs) to `out` (32 values) and clears them.  Synchronises the device.
+extern "C" int sage_tile_timing(unsigned long long* out) {
+  static const unsigned long long zero[32] = {};
+  if (hipDeviceSynchronize() != hipSuccess) return -1;
+  if (hipMemcpyFromSymbol(out, HIP_SYMBOL(sage::g_tile_timing), sizeof(zero)) != hipSuccess) return -1;
+  return hipMemcpyToSymbol(HIP_SYMBOL(sage::g_tile_timing), zero, sizeof(zero)) == hipSuccess ? 0 : -1;
 }
 #endif

@@ -4,6 +4,7 @@ What it mirrors: the 20-shape table, the custom-shape options, the validation ru
 backends/_enflame/benchmarks/sage_attention_native_benchmark.py:70-78, :158-198, :447-455.
 """
 import json
+import os
 
 import pytest
 
@@ -79,3 +80,26 @@ def test_hw_rate_microbenchmarks_run_and_are_plausible():
             best[r["kind"]] = max(best.get(r["kind"], 0.0), r["chip_TOPS"])
     assert best[0] > 2500 and best[1] > 2500, best
     assert best[3] <= best[0] * 1.05 and best[4] <= best[1] * 1.05, best   # feeding from LDS never beats registers
+
+
+@pytest.mark.gpu
+def test_tile_timing_tool_reports_the_intervals_of_a_workgroup():
+    """The instrumented twin of the library, loaded in its own process through SAGE_MI355X_LIB: every interval
+    of a workgroup is positive and the main loop dominates a 4k-key causal tile."""
+    import subprocess
+    import sys
+    from baselinebenchmark_amd.build import TIMING_LIB
+    ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    if not TIMING_LIB.exists():
+        pytest.skip("timing build absent (python -m baselinebenchmark_amd.build --timing)")
+    code = ("from baselinebenchmark_amd.benchmarks import tile_timing as t\n"
+            "rows, tiles = t.measure(2, 4, 4096, 128, True, launches=2)\n"
+            "import json; print(json.dumps({'rows': rows, 'tiles': tiles}))\n")
+    env = dict(os.environ, SAGE_MI355X_LIB=str(TIMING_LIB))
+    res = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, env=env, cwd=ROOT, timeout=240)
+    assert res.returncode == 0, res.stderr[-2000:]
+    doc = json.loads([l for l in res.stdout.splitlines() if l.startswith("{")][-1])
+    assert abs(doc["tiles"] - 17.0) < 1e-6          # 16 q-tiles of 256 rows: 2, 4, ..., 32 K tiles of 128 keys
+    for name, vals in doc["rows"].items():
+        assert len(vals) == 7 and all(v > 0 for v in vals), (name, vals)
+        assert vals[4] > 0.5 * sum(vals), (name, vals)
