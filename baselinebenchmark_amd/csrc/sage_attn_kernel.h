@@ -86,11 +86,15 @@ __device__ inline int kswz(int n) {
   return (n / RPB) % CPR;
 }
 
-// LDS slots per tile stream = how far ahead tiles are requested (slots - 1 periods before their first
-// use).  Two periods pay where every q-tile streams the whole sequence (non-causal, FP8 P.V: +4...7 %
-// measured from 1k to 16k keys); for causal and FP16 P.V kernels one period measured 1-3 % faster.
+// LDS slots per tile stream.  FP8 P.V kernels rotate through four and request tiles two periods before
+// their first use (a tile that has to come from HBM takes longer than one 2 us period: +5...8 % for
+// non-causal kernels from 1k to 16k keys, neutral for causal ones; three slots measured 1-2 % slower
+// than four, the slot index being a modulo in the loop).  FP16 P.V tiles are twice as large: two
+// slots, one period (three slots measured 1-3 % slower there).
 template <int PV, bool CAUSAL>
-constexpr int attn_tile_slots() { return (PV == 1 && !CAUSAL) ? 3 : 2; }
+constexpr int attn_tile_slots() { return PV == 1 ? 4 : 2; }
+template <int PV, bool CAUSAL>
+constexpr int attn_tile_lead() { return attn_tile_slots<PV, CAUSAL>() > 2 ? 2 : 1; }
 
 // Dynamic LDS of a kernel variant: the K slots and as many V slots; a kernel that quantises its own Q also
 // stages the raw q-tile behind the K slots that are requested in the prologue (over slots that are idle
@@ -99,7 +103,7 @@ template <int D, int NW, int BN, int PV, bool CAUSAL, bool QF>
 constexpr int attn_tile_lds_bytes() {
   constexpr int slots = attn_tile_slots<PV, CAUSAL>();
   constexpr int tiles = slots * (BN * D + BN * D * (PV ? 1 : 2));
-  constexpr int qstage = (slots - 1) * BN * D + NW * 32 * D * 2;
+  constexpr int qstage = attn_tile_lead<PV, CAUSAL>() * BN * D + NW * 32 * D * 2;
   return (QF && qstage > tiles) ? qstage : tiles;
 }
 template <int D, int NW, int BN, int PV, bool CAUSAL, bool QF>
@@ -134,7 +138,7 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
   constexpr int PANEL_BYTES = kPanelRows * D * VESZ;
   constexpr int CPR = D / 16;
   constexpr float TAU = PCfg<PV>::tau, PSHIFT = PCfg<PV>::pshift;
-  constexpr int NSLOT = attn_tile_slots<PV, CAUSAL>(), LEAD = NSLOT - 1;   // tiles are requested LEAD periods ahead
+  constexpr int NSLOT = attn_tile_slots<PV, CAUSAL>(), LEAD = attn_tile_lead<PV, CAUSAL>();   // tiles are requested LEAD periods ahead
 
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
