@@ -692,11 +692,16 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
     constexpr int UPR = D / 8;        // 16-byte units per output row
     constexpr int RPI = 64 / UPR;     // rows per store instruction
     uint8_t* stage = smem + w * (32 * D * 2);
+    // The lane index is made opaque here: addresses derived from it are then computed now, not before the
+    // main loop, where they would be parked in scratch memory for its duration.
+    int el = lane;
+    asm volatile("" : "+v"(el));
+    const int em = el & 31, eh = el >> 5;
 #pragma unroll
     for (int dt = 0; dt < DTN; dt++) {
 #pragma unroll
       for (int q4 = 0; q4 < 4; q4++) {
-        const int d = 32 * dt + 8 * q4 + 4 * h;
+        const int d = 32 * dt + 8 * q4 + 4 * eh;
         float f[4];
 #pragma unroll
         for (int i = 0; i < 4; i++) {
@@ -708,10 +713,10 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
         for (int i = 0; i < 4; i++) hv[i] = a.out_bf16 ? f32_to_bf16(f[i]) : f32_to_f16(f[i]);
         uint2 pkd = make_uint2((uint32_t)hv[0] | ((uint32_t)hv[1] << 16), (uint32_t)hv[2] | ((uint32_t)hv[3] << 16));
         const int u = 4 * dt + q4;    // 16-byte unit of the row; h picks its half
-        *reinterpret_cast<uint2*>(stage + m * (D * 2) + ((u ^ (m & (UPR - 1))) * 16) + 8 * h) = pkd;
+        *reinterpret_cast<uint2*>(stage + em * (D * 2) + ((u ^ (em & (UPR - 1))) * 16) + 8 * eh) = pkd;
       }
     }
-    const int k16 = lane % UPR, rsub = lane / UPR;
+    const int k16 = el % UPR, rsub = el / UPR;
 #pragma unroll
     for (int i = 0; i < 32 / RPI; i++) {
       const int r = i * RPI + rsub;
