@@ -30,9 +30,9 @@ PEAK_FP16 = 2516.6       # dense FP16 MFMA peak, TFLOP/s
 
 
 # HBM-side bytes per launch of the attention kernel, from the committed rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# runs on this same command (profiles/attn_kernel_c2_pmc.md): (1 245 740 + 262 513) counter units x 2.0 (the factor the
+# runs on this same command (profiles/attn_kernel_c2_pmc.md): (1 245 800 + 262 140) counter units x 2.0 (the factor the
 # same counters read for a 512 MiB device copy) x 1 KiB.  Measured for config 2 only.
-TRAFFIC_BYTES = {"c2": (1245740 + 262420) * 2.0 * 1024}
+TRAFFIC_BYTES = {"c2": (1245800 + 262140) * 2.0 * 1024}
 
 
 def blended_peak(pv: str) -> float:
