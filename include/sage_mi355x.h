@@ -134,7 +134,9 @@ int sage_varlen_plan(const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k, i
  * q_scale/k_scale: as written by sage_quant_int8 with blkq in {32, 64, 128}, blkk in {16, 32, 64, 128}
  * (16: the K granularity of the external recipe (128, 16), sage_attention_benchmark_compare.py:93).
  * v_panels/v_scale: as written by sage_prep_v (v_scale NULL for SAGE_PV_FP16).
- * out: fp16/bf16 (out_dtype) addressed with (o_sb,o_sh,o_sn); lse may be NULL.
+ * out: fp16/bf16 (out_dtype) addressed with (o_sb,o_sh,o_sn), base and strides multiples of 16 bytes (rows are
+ * stored 16 bytes per lane); lse may be NULL.  A (batch, head) slice of k -- and of a floating-point q in
+ * sage_attn_fwd_qfused -- must span less than 2 GiB (tile loads use 32-bit byte offsets): SAGE_ENOTIMPL otherwise.
  * Packed mode: cu_seqlens_q != NULL; B = nseq, Sq/Skv = longest sequences, `plan` from
  * sage_varlen_plan, total_q = number of packed query rows, scale/panel head strides given.
  */
