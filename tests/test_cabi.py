@@ -83,6 +83,19 @@ def test_attn_argument_errors(sage_lib):
     assert call(pv=5) == _cabi.SAGE_EINVAL
 
 
+def test_attn_alignment_and_slice_limits(sage_lib):
+    def call(out=FAKE, o_sn=128, Skv=128, k_sn=128):
+        return sage_lib.sage_attn_fwd(FAKE, FAKE, FAKE, FAKE, FAKE, NULL, out, NULL, 1, 4, 2, 128, Skv, 128,
+                                      0, 128 * 128, 128, 0, 128 * 128, k_sn, 0, 128 * 128, o_sn, 128, 64, 0, 0, 0,
+                                      NULL, NULL, NULL, 0, 0, 0, 0, NULL)
+    assert call(out=ctypes.c_void_p(4096 + 8)) == _cabi.SAGE_EINVAL     # rows are stored 16 bytes per lane
+    assert call(o_sn=100) == _cabi.SAGE_EINVAL                          # 200-byte row stride
+    assert "16-byte" in sage_lib.sage_last_error().decode()
+    # tile loads address a (batch, head) slice of k with 32-bit byte offsets
+    assert call(Skv=1 << 20, k_sn=4096) == _cabi.SAGE_ENOTIMPL
+    assert "2 GiB" in sage_lib.sage_last_error().decode()
+
+
 def test_empty_problem_is_a_no_op(sage_lib):
     rc = sage_lib.sage_quant_int8(NULL, NULL, NULL, NULL, 0, 4, 128, 128, 0, 0, 128, 0, 0, 128, 0, 0, 128, 1.0, 0,
                                   NULL, NULL, 0, NULL)
