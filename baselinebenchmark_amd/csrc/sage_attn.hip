@@ -42,10 +42,28 @@ __global__ void __launch_bounds__(1024) varlen_plan_kernel(const int32_t* cu_q, 
     for (int qt = tid; qt < nqt; qt += blockDim.x) atomicAdd(&hist[cost_of(lq, lk, qt)], 1);
   }
   __syncthreads();
-  if (tid == 0) {
-    int acc = 0;
-    for (int c = kCostBins - 1; c >= 0; c--) { start[c] = acc; acc += hist[c]; }
-    plan[L.ntiles] = acc;
+  // start[c] = number of tiles in more expensive bins: an exclusive scan over the bins in descending cost
+  // order, two bins per thread, wavefront scans combined through LDS.
+  {
+    static_assert(kCostBins == 2048, "two bins per thread of a 1024-thread workgroup");
+    __shared__ int wave_total[16];
+    const int c0 = kCostBins - 1 - 2 * tid, c1 = c0 - 1;   // this thread's bins, the more expensive one first
+    const int h0 = hist[c0], h1 = hist[c1];
+    int incl = h0 + h1;
+    const int lane = tid & 63, wv = tid >> 6;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int up = __shfl_up(incl, d, 64);
+      if (lane >= d) incl += up;
+    }
+    if (lane == 63) wave_total[wv] = incl;
+    __syncthreads();
+    int before = 0;
+    for (int i = 0; i < wv; i++) before += wave_total[i];
+    const int excl = before + incl - (h0 + h1);
+    start[c0] = excl;
+    start[c1] = excl + h0;
+    if (tid == 1023) plan[L.ntiles] = before + incl;
   }
   __syncthreads();
   // pass 2: place tiles, most expensive bins first
