@@ -1,0 +1,69 @@
+"""Seeded random configurations through the whole public surface, each checked three ways: the INT8 operands and
+the K mean bit-exact against the oracle's quantiser (quant_per_block.py:38-46), `forward` against the reference
+formula on the same quantised operands (test_sageattention_hip.py:12-28; FP16 P.V: relative RMSE, FP8 P.V:
+cosine >= 0.999), and the one-call `sageattn` bit-identical to `forward` and within cosine 0.998 of FP32 SDPA on
+the raw inputs.  Shapes mix head dims, layouts, GQA ratios, ragged lengths, scale-block sizes and both P.V modes."""
+import random
+
+import pytest
+import torch
+
+import baselinebenchmark_amd as sa
+from oracle import attention as oa
+from oracle import quant as oq
+
+pytestmark = [pytest.mark.gpu, pytest.mark.sage_attention]
+DEV = "cuda"
+LENGTHS = [1, 7, 31, 64, 100, 128, 129, 255, 256, 257, 300, 511, 513, 700, 1025]
+
+
+def _draw(rng):
+    c = dict(D=rng.choice([64, 128]), dtype=rng.choice([torch.float16, torch.bfloat16]), layout=rng.choice(["HND", "NHD"]),
+             Hkv=rng.choice([1, 2, 3, 8]), G=rng.choice([1, 1, 2, 4]), B=rng.choice([1, 1, 2, 3]), S=rng.choice(LENGTHS),
+             causal=rng.random() < 0.5, pv=rng.choice(["fp16", "fp8"]), blkq=rng.choice([32, 64, 128]),
+             blkk=rng.choice([16, 32, 64, 128]), smooth=rng.random() < 0.7, lse=rng.random() < 0.3, seed=rng.randrange(1 << 30))
+    c["Skv"] = c["S"] if (c["causal"] or rng.random() < 0.5) else rng.choice([1, 5, 64, 130, 260, 777])
+    return c
+
+
+CASES = [_draw(random.Random(1000 + i)) for i in range(48)]
+
+
+@pytest.mark.parametrize("c", CASES, ids=[f"case{i}" for i in range(len(CASES))])
+def test_random_configuration(c):
+    D, dtype, layout, B, Hkv, S, Skv = c["D"], c["dtype"], c["layout"], c["B"], c["Hkv"], c["S"], c["Skv"]
+    Hq = Hkv * c["G"]
+    g = torch.Generator().manual_seed(c["seed"])
+    shape = (lambda H, L: (B, H, L, D)) if layout == "HND" else (lambda H, L: (B, L, H, D))
+    q = torch.randn(shape(Hq, S), generator=g).to(dtype)
+    k = (torch.randn(shape(Hkv, Skv), generator=g) + 1.0).to(dtype)
+    v = torch.randn(shape(Hkv, Skv), generator=g).to(dtype)
+    qd, kd, vd = q.to(DEV), k.to(DEV), v.to(DEV)
+    blk = dict(BLKQ=c["blkq"], BLKK=c["blkk"])
+
+    km = sa.k_mean(kd, layout) if c["smooth"] else None
+    km_ref = oq.k_mean(k, layout) if c["smooth"] else None
+    if c["smooth"]:
+        assert torch.equal(km.cpu().view(torch.int16), km_ref.view(torch.int16))
+    qi, qs, ki, ks = sa.per_block_int8(qd, kd, km=km, tensor_layout=layout, **blk)
+    rqi, rqs, rki, rks = oq.per_block_int8(q, k, km=km_ref, tensor_layout=layout, **blk)
+    assert torch.equal(qi.cpu(), rqi) and torch.equal(ki.cpu(), rki)
+    assert torch.equal(qs.cpu(), rqs) and torch.equal(ks.cpu(), rks)
+
+    out, lse2 = sa.forward(qi, ki, vd, qs, ks, tensor_layout=layout, output_dtype=dtype, return_lse=c["lse"],
+                           is_causal=c["causal"], pv_mode=c["pv"], **blk)
+    ref, ref_lse = oa.sage_reference(qi.cpu(), ki.cpu(), v, qs.cpu(), ks.cpu(), layout, c["blkq"], c["blkk"], is_causal=c["causal"])
+    m = oa.metrics(out.cpu().float(), ref)
+    assert m["finite"]
+    if c["pv"] == "fp16":
+        assert m["rel_rmse"] < (6e-3 if dtype == torch.bfloat16 else 2e-3), m     # output rounding of the dtype
+    else:
+        assert m["cosine"] >= 0.999, m
+    if c["lse"]:
+        assert (lse2.cpu().double() - ref_lse).abs().max().item() < (1e-3 if c["pv"] == "fp16" else 5e-2)
+
+    one = sa.sageattn(qd, kd, vd, tensor_layout=layout, is_causal=c["causal"], smooth_k=c["smooth"], pv_mode=c["pv"], **blk)
+    if not c["lse"]:     # with LSE `forward` keeps the FP32 row sums: a different (more accurate) denominator
+        assert torch.equal(one, out)
+    m2 = oa.metrics(one.cpu().float(), oa.sdpa_fp32(q, k, v, layout, c["causal"]))
+    assert m2["finite"] and m2["cosine"] >= 0.998, m2
