@@ -84,3 +84,27 @@ def test_config4_full_size_sequences_are_independent():
         alone = sa.sageattn(w.q[sl].unsqueeze(0).contiguous(), w.k[sl].unsqueeze(0).contiguous(), w.v[sl].unsqueeze(0).contiguous(),
                             tensor_layout="NHD", **w.kwargs)
         assert torch.equal(out[sl], alone[0]), (i, lens[i])
+
+
+def _draw_packed(rng):
+    lens_pool = [1, 2, 31, 64, 127, 128, 129, 255, 256, 257, 300, 513, 700, 1030]
+    hkv = rng.choice([1, 2, 8])
+    return dict(D=rng.choice([64, 128]), dtype=rng.choice([torch.float16, torch.bfloat16]), Hkv=hkv, Hq=hkv * rng.choice([1, 2, 4]),
+                lens=[rng.choice(lens_pool) for _ in range(rng.choice([1, 2, 3, 6, 9]))], causal=rng.random() < 0.5,
+                pv=rng.choice(["fp16", "fp8"]), blkq=rng.choice([32, 64, 128]), blkk=rng.choice([32, 64, 128]),
+                smooth=rng.random() < 0.7, seed=rng.randrange(1 << 30))
+
+
+@pytest.mark.parametrize("c", [_draw_packed(__import__("random").Random(500 + i)) for i in range(16)], ids=[f"case{i}" for i in range(16)])
+def test_random_packed_batches_match_sdpa_and_the_fixed_length_call(c):
+    q, k, v, cu = _packed(c["lens"], c["Hq"], c["Hkv"], c["D"], c["dtype"], c["seed"])
+    kw = dict(is_causal=c["causal"], pv_mode=c["pv"], BLKQ=c["blkq"], BLKK=c["blkk"], smooth_k=c["smooth"])
+    qd, kd, vd = q.to(DEV), k.to(DEV), v.to(DEV)
+    out = sa.sageattn_varlen(qd, kd, vd, cu.to(DEV), cu.to(DEV), max(c["lens"]), max(c["lens"]), **kw)
+    ref = oa.sdpa_fp32_varlen(q, k, v, cu, cu, c["causal"])
+    for i in range(len(c["lens"])):
+        a, b = int(cu[i]), int(cu[i + 1])
+        m = oa.metrics(out[a:b].cpu().float(), ref[a:b])
+        assert m["finite"] and m["cosine"] >= 0.998, (i, c["lens"][i], m)
+        one = sa.sageattn(qd[a:b].unsqueeze(0), kd[a:b].unsqueeze(0), vd[a:b].unsqueeze(0), tensor_layout="NHD", **kw)
+        assert torch.equal(one[0], out[a:b]), (i, c["lens"][i])
