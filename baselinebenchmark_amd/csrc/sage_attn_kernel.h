@@ -742,14 +742,18 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
 
 template <int D, int NW, int BN, int PV, bool CAUSAL, bool MSUM, int MASK, int KSUB = 1, bool QF = false>
 static hipError_t launch_one(const AttnArgs& a, int grid, hipStream_t st) {
-  constexpr int VESZ = PV ? 1 : 2;
   constexpr int smem = attn_lds_bytes<D, NW, BN, PV, CAUSAL, QF>();
   auto kern = attn_kernel<D, NW, BN, PV, CAUSAL, MSUM, MASK, KSUB, QF>;
-  static bool attr_done = false;
-  if (!attr_done) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+  // More than 64 KB of dynamic LDS has to be allowed once per kernel and device.
+  constexpr int kMaxDevices = 64;
+  static bool attr_done[kMaxDevices] = {};
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (dev < 0 || dev >= kMaxDevices || !attr_done[dev]) {
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return e;
-    attr_done = true;
+    if (dev >= 0 && dev < kMaxDevices) attr_done[dev] = true;
   }
   kern<<<dim3(grid), dim3(NW * 64), smem, st>>>(a);
   return hipGetLastError();
