@@ -311,8 +311,25 @@ def forward_fused_q(q, k, v, k_scale, tensor_layout="HND", sm_scale=None, output
 # ------------------------------------------------------------------------------------------------
 # one-call API
 # ------------------------------------------------------------------------------------------------
+def _apply_recipe(quant_recipe, BLKQ, BLKK, pv_mode):
+    """``quant_recipe`` as passed at sage_attention_benchmark_compare.py:93, :300-313 -- (Q rows per scale, K rows
+    per scale, V rows per scale with -1 = the whole sequence, V channels per scale): the one V granularity built
+    here is (-1, 1), per-channel FP8-e4m3 V (``V=FP8``, :571), so a recipe selects the FP8 P.V path."""
+    if quant_recipe is None:
+        return BLKQ, BLKK, ("fp16" if pv_mode is None else pv_mode)
+    try:
+        bq, bk, vrows, vcols = (int(x) for x in quant_recipe)
+    except (TypeError, ValueError) as exc:
+        raise ValueError(f"quant_recipe must be four integers, got {quant_recipe!r}") from exc
+    if (vrows, vcols) != (-1, 1):
+        raise NotImplementedError("V is quantised per channel over the whole sequence: quant_recipe[2:] must be (-1, 1)")
+    if pv_mode is not None and _pv(pv_mode) != PV_FP8:
+        raise ValueError("a quant_recipe quantises V to FP8: pv_mode must be 'fp8' or left unset")
+    return bq, bk, "fp8"
+
+
 @torch.no_grad()
-def sageattn(q, k, v, tensor_layout="HND", is_causal=False, sm_scale=None, smooth_k=True, pv_mode="fp16",
+def sageattn(q, k, v, tensor_layout="HND", is_causal=False, sm_scale=None, smooth_k=True, pv_mode=None,
              BLKQ=128, BLKK=64, return_lse=False, qk_quant_dtype="int8", quant_recipe=None, attn_mask=None, **kwargs):
     """Quantise + attend in one call: out = softmax(q k^T * sm_scale [causal | + attn_mask]) v.
 
@@ -321,11 +338,15 @@ def sageattn(q, k, v, tensor_layout="HND", is_causal=False, sm_scale=None, smoot
     removes from the logits is added back (checked as in test_sage_attention_mate.py:171-178).
     ``attn_mask``: boolean (True keeps) or additive in natural-log units, broadcastable to
     [B, Hq, Sq, Skv]; not combinable with ``is_causal``.
+    ``quant_recipe`` (the keyword of sage_attention_benchmark_compare.py:300-313): (Q rows, K rows, -1, 1) sets the
+    scale blocks and selects per-channel FP8 V, e.g. the external recipe (128, 16, -1, 1); without it ``BLKQ`` /
+    ``BLKK`` / ``pv_mode`` ("fp16" by default) apply.
     """
     if qk_quant_dtype != "int8":
         raise NotImplementedError("only INT8 Q/K quantisation is implemented")
     if kwargs:
         raise TypeError(f"unexpected arguments: {sorted(kwargs)}")
+    BLKQ, BLKK, pv_mode = _apply_recipe(quant_recipe, BLKQ, BLKK, pv_mode)
     for name, t in (("q", q), ("k", k), ("v", v)):
         _check_float(name, t)
     if not (q.dtype == k.dtype == v.dtype) or not (q.device == k.device == v.device):

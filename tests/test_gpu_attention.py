@@ -347,3 +347,19 @@ def test_config3_full_size_properties():
     start = (S // 256) * 256
     tail = sa.sageattn(w.q[:, start:].contiguous(), w.k, w.v, **w.kwargs)
     assert torch.equal(tail, out[:, start:])
+
+
+def test_sageattn_with_the_external_quant_recipe():
+    """The call of sage_attention_benchmark_compare.py:300-313: quant_recipe=(128, 16, -1, 1), smooth_k=True, INT8 Q/K,
+    FP8 V.  Same result as naming the blocks and the P.V mode directly, and within the north-star gate of FP32 SDPA."""
+    g = torch.Generator().manual_seed(77)
+    q = randn("HND", 2, 8, 1000, 128, torch.float16, g)
+    k = randn("HND", 2, 8, 1000, 128, torch.float16, g) + 1.0
+    v = randn("HND", 2, 8, 1000, 128, torch.float16, g)
+    qd, kd, vd = q.to(DEV), k.to(DEV), v.to(DEV)
+    out = sa.sageattn(qd, kd, vd, tensor_layout="HND", is_causal=False, qk_quant_dtype="int8", quant_recipe=(128, 16, -1, 1),
+                      smooth_k=True, return_lse=False)
+    same = sa.sageattn(qd, kd, vd, tensor_layout="HND", is_causal=False, BLKQ=128, BLKK=16, pv_mode="fp8", smooth_k=True)
+    assert torch.equal(out, same)
+    m = oa.metrics(out.cpu().float(), oa.sdpa_fp32(q, k, v, "HND", False))
+    assert m["finite"] and m["cosine"] >= 0.999, m

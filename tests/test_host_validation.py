@@ -93,6 +93,15 @@ def test_sageattn_contract():
         sa.sageattn(q, k, k, tensor_layout="NHD", bogus=1)
     with pytest.raises(ValueError):
         sa.sageattn(fake(1, 128, 3, 128), k, k, tensor_layout="NHD")
+    # quant_recipe as passed at sage_attention_benchmark_compare.py:300-313: (Q rows, K rows, -1, 1) -> FP8 V
+    with pytest.raises(ValueError):
+        sa.sageattn(q, k, k, tensor_layout="NHD", quant_recipe=(128, 16))
+    with pytest.raises(NotImplementedError):
+        sa.sageattn(q, k, k, tensor_layout="NHD", quant_recipe=(128, 16, 64, 1))
+    with pytest.raises(ValueError):
+        sa.sageattn(q, k, k, tensor_layout="NHD", quant_recipe=(128, 16, -1, 1), pv_mode="fp16")
+    with pytest.raises(NotImplementedError):
+        sa.sageattn(q, k, k, tensor_layout="NHD", quant_recipe=(128, 8, -1, 1))      # K blocks: 16 rows or more
 
 
 def test_varlen_contract():
