@@ -215,7 +215,7 @@ int attn_impl(const int8_t* q, const int8_t* k, const void* v_panels, const floa
   if (B == 0 || Hq == 0 || Sq == 0) return SAGE_OK;
   if (!k || !v_panels || !k_scale || !out) return fail(SAGE_EINVAL, "null tensor pointer");
   if (!qraw.ptr && (!q || !q_scale)) return fail(SAGE_EINVAL, "null tensor pointer");
-  if (qraw.ptr && (mask.ptr || blkk == 16)) return fail(SAGE_ENOTIMPL, "fused Q quantisation: not with a mask or K blocks of 16");
+  if (qraw.ptr && mask.ptr) return fail(SAGE_ENOTIMPL, "fused Q quantisation: not with an explicit mask");
   if (pv_mode == SAGE_PV_FP8 && !v_scale) return fail(SAGE_EINVAL, "fp8 P.V needs v_scale");
   if (int rc = check_stride16("q", q_sb, q_sh, q_sn, qraw.ptr ? 2 : 1, qraw.ptr ? qraw.ptr : q)) return rc;
   if (int rc = check_stride16("k", k_sb, k_sh, k_sn, 1, k)) return rc;
@@ -414,9 +414,9 @@ int sage_sageattn_masked(const void* q, const void* k, const void* v, void* out,
     dot.vec = km; dot.out = lse_off; dot.sb = (int64_t)Hkv * D; dot.sh = D; dot.group = Hq / Hkv; dot.total = total_q;
   }
   // Q is quantised by the attention kernel itself (each q-tile exactly where it is consumed) unless a
-  // feature needs the standalone pass: an explicit mask, K blocks of 16, or the LSE correction.
+  // feature needs the standalone pass: an explicit mask or the LSE correction.
   const float q_mult = (float)((sm_scale > 0 ? sm_scale : 1.0 / sqrt((double)D)) * 1.44269504);
-  const bool fuse_q = !attn_mask && blkk != 16 && !lse_off;
+  const bool fuse_q = !attn_mask && !lse_off;
   if (!fuse_q) {
     rc = quant_impl(q, q_i8, q_scale, nullptr, B, Hq, Sq, D, q_sb, q_sh, q_sn, q_sb, q_sh, q_sn, 0, 0, blkq, q_mult, dtype,
                     cu_seqlens_q, cu_qblk, w.qs_sh, dot, stream);

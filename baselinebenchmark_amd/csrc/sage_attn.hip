@@ -91,8 +91,8 @@ AttnConfig attn_config(int D, int pv, bool packed) {
 hipError_t launch_attn(const AttnArgs& a, int D, int pv, bool causal, int grid, hipStream_t st) {
   if (grid == 0) return hipSuccess;
   if (a.mask) return launch_attn_masked(a, D, pv, grid, st);
-  if (a.q_raw) return launch_attn_qfused(a, D, pv, causal, grid, st);
   if (a.blkk == 16) return launch_attn_k16(a, D, pv, causal, grid, st);
+  if (a.q_raw) return launch_attn_qfused(a, D, pv, causal, grid, st);
   const bool msum = pv && a.lse == nullptr;   // row sums on the matrix pipe unless LSE is wanted
 #define SAGE_ATTN(DD, PVV, BNN, MS) (causal ? launch_one<DD, 8, BNN, PVV, true, MS, 0>(a, grid, st) : launch_one<DD, 8, BNN, PVV, false, MS, 0>(a, grid, st))
   if (D == 128) return pv ? (msum ? SAGE_ATTN(128, 1, 128, true) : SAGE_ATTN(128, 1, 128, false)) : SAGE_ATTN(128, 0, 128, false);

@@ -15,10 +15,15 @@ hipError_t launch_attn_masked(const AttnArgs& a, int D, int pv, int grid, hipStr
 }
 
 hipError_t launch_attn_k16(const AttnArgs& a, int D, int pv, bool causal, int grid, hipStream_t st) {
-#define SAGE_ATTN_K(DD, PVV, BNN) (causal ? launch_one<DD, 8, BNN, PVV, true, false, 0, 2>(a, grid, st) : launch_one<DD, 8, BNN, PVV, false, false, 0, 2>(a, grid, st))
-  if (D == 128) return pv ? SAGE_ATTN_K(128, 1, 128) : SAGE_ATTN_K(128, 0, 128);
-  return pv ? SAGE_ATTN_K(64, 1, 128) : SAGE_ATTN_K(64, 0, 128);
+  // Row sums on the matrix pipe for FP8 P.V without LSE, as for the coarser K blocks; with a floating-point
+  // Q (a.q_raw) the q-tile is quantised in the prologue.
+  const bool msum = pv && a.lse == nullptr;
+#define SAGE_ATTN_KQ(DD, PVV, MS, QFF) (causal ? launch_one<DD, 8, 128, PVV, true, MS, 0, 2, QFF>(a, grid, st) : launch_one<DD, 8, 128, PVV, false, MS, 0, 2, QFF>(a, grid, st))
+#define SAGE_ATTN_K(DD, PVV, MS) (a.q_raw ? SAGE_ATTN_KQ(DD, PVV, MS, true) : SAGE_ATTN_KQ(DD, PVV, MS, false))
+  if (D == 128) return pv ? (msum ? SAGE_ATTN_K(128, 1, true) : SAGE_ATTN_K(128, 1, false)) : SAGE_ATTN_K(128, 0, false);
+  return pv ? (msum ? SAGE_ATTN_K(64, 1, true) : SAGE_ATTN_K(64, 1, false)) : SAGE_ATTN_K(64, 0, false);
 #undef SAGE_ATTN_K
+#undef SAGE_ATTN_KQ
 }
 
 }  // namespace sage

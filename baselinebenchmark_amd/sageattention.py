@@ -290,8 +290,8 @@ def forward_fused_q(q, k, v, k_scale, tensor_layout="HND", sm_scale=None, output
         raise ValueError("query heads must be divisible by KV heads")
     if D not in (64, 128):
         raise NotImplementedError("head_dim must be 64 or 128")
-    if BLKQ not in (32, 64, 128) or BLKK not in (32, 64, 128):
-        raise NotImplementedError("the fused-Q kernel needs scale blocks of 32, 64 or 128 rows")
+    if BLKQ not in (32, 64, 128) or BLKK not in (16, 32, 64, 128):
+        raise NotImplementedError("the fused-Q kernel needs Q scale blocks of 32/64/128 and K scale blocks of 16/32/64/128 rows")
     if tuple(k_scale.shape) != (B, Hkv, (Skv + BLKK - 1) // BLKK):
         raise ValueError(f"k_scale has shape {tuple(k_scale.shape)}, expected {(B, Hkv, (Skv + BLKK - 1) // BLKK)}")
     pv = _pv(pv_mode)

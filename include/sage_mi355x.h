@@ -203,7 +203,7 @@ int sage_attn_fwd_masked(const int8_t* q, const int8_t* k, const void* v_panels,
  * entry point exercised at backends/_metax/benchmarks/sage_attention/benchmark.py:29 and
  * backends/_mthreads/benchmarks/sage_attention_benchmark_compare.py:300-313:
  * [K mean] -> quantise K (minus mean) -> prepare V -> attention (which quantises its own Q tiles; a
- * separate Q pass only where a mask, K blocks of 16 rows or the LSE correction need one).
+ * separate Q pass only where a mask or the LSE correction need one).
  * All intermediates live in `workspace` (sage_sageattn_workspace_bytes); nothing is allocated.
  * smooth_k != 0 subtracts the per-channel K mean.  sm_scale <= 0 selects head_dim^-0.5; the Q
  * multiplier is (float)(sm_scale * 1.44269504), the double product of quant_per_block.py:87.  Packed mode as in sage_attn_fwd

@@ -292,7 +292,13 @@ def test_forward_fused_q_entry_point_matches_quantise_then_forward_bitwise():
     with pytest.raises(TypeError):
         sa.forward_fused_q(qi, ki, v, ks)          # q must be floating point
     with pytest.raises(NotImplementedError):
-        sa.forward_fused_q(q, ki, v, ks, BLKK=16)
+        sa.forward_fused_q(q, ki, v, ks, BLKK=8)
+    # K scale blocks of 16 rows (two scales per 32-key MFMA tile): the same identity
+    qi, qs, ki, ks = sa.per_block_int8(q, k, BLKQ=128, BLKK=16)
+    for lse in (False, True):
+        a, la = sa.forward(qi, ki, v, qs, ks, output_dtype=torch.bfloat16, BLKQ=128, BLKK=16, pv_mode="fp8", return_lse=lse)
+        b, lb = sa.forward_fused_q(q, ki, v, ks, BLKQ=128, BLKK=16, pv_mode="fp8", return_lse=lse)
+        assert torch.equal(a, b) and torch.equal(la, lb)
 
 
 def test_config2_full_size_properties():
