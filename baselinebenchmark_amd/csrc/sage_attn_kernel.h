@@ -697,25 +697,31 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
     int el = lane;
     asm volatile("" : "+v"(el));
     const int em = el & 31, eh = el >> 5;
+    // (one copy of the loop per output type: the type is uniform, and converting both ways and selecting
+    // per element would double the conversions)
+    auto normalise_and_stage = [&](auto to_out) {
 #pragma unroll
-    for (int dt = 0; dt < DTN; dt++) {
+      for (int dt = 0; dt < DTN; dt++) {
 #pragma unroll
-      for (int q4 = 0; q4 < 4; q4++) {
-        const int d = 32 * dt + 8 * q4 + 4 * eh;
-        float f[4];
+        for (int q4 = 0; q4 < 4; q4++) {
+          const int d = 32 * dt + 8 * q4 + 4 * eh;
+          float f[4];
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-          f[i] = o[dt][4 * q4 + i] * inv;
-          if constexpr (PV == 1) f[i] *= vs_lds[d + i];
+          for (int i = 0; i < 4; i++) {
+            f[i] = o[dt][4 * q4 + i] * inv;
+            if constexpr (PV == 1) f[i] *= vs_lds[d + i];
+          }
+          u16 hv[4];
+#pragma unroll
+          for (int i = 0; i < 4; i++) hv[i] = to_out(f[i]);
+          uint2 pkd = make_uint2((uint32_t)hv[0] | ((uint32_t)hv[1] << 16), (uint32_t)hv[2] | ((uint32_t)hv[3] << 16));
+          const int u = 4 * dt + q4;    // 16-byte unit of the row; h picks its half
+          *reinterpret_cast<uint2*>(stage + em * (D * 2) + ((u ^ (em & (UPR - 1))) * 16) + 8 * eh) = pkd;
         }
-        u16 hv[4];
-#pragma unroll
-        for (int i = 0; i < 4; i++) hv[i] = a.out_bf16 ? f32_to_bf16(f[i]) : f32_to_f16(f[i]);
-        uint2 pkd = make_uint2((uint32_t)hv[0] | ((uint32_t)hv[1] << 16), (uint32_t)hv[2] | ((uint32_t)hv[3] << 16));
-        const int u = 4 * dt + q4;    // 16-byte unit of the row; h picks its half
-        *reinterpret_cast<uint2*>(stage + em * (D * 2) + ((u ^ (em & (UPR - 1))) * 16) + 8 * eh) = pkd;
       }
-    }
+    };
+    if (a.out_bf16) normalise_and_stage([](float x) { return f32_to_bf16(x); });
+    else normalise_and_stage([](float x) { return f32_to_f16(x); });
     const int k16 = el % UPR, rsub = el / UPR;
 #pragma unroll
     for (int i = 0; i < 32 / RPI; i++) {
