@@ -50,7 +50,7 @@ def build_parser() -> argparse.ArgumentParser:
     p.add_argument("--dtype", choices=TABLE_DTYPES, default="float16")
     p.add_argument("--causal", action="store_true", help="causal mask (effective ops are halved)")
     p.add_argument("--pv", choices=("fp16", "fp8"), default="fp16", help="precision of the P.V product")
-    p.add_argument("--blkq", type=int, choices=(32, 64, 128), default=128)
+    p.add_argument("--blkq", type=int, choices=(16, 32, 64, 128), default=128)
     p.add_argument("--blkk", type=int, choices=(16, 32, 64, 128), default=64)
     p.add_argument("--warmup", type=int, default=5)
     p.add_argument("--rep", type=int, default=20)

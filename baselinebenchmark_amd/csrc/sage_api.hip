@@ -31,8 +31,8 @@ int hip_fail(hipError_t e, const char* what) {
 inline size_t align_up(size_t x, size_t a = 256) { return (x + a - 1) / a * a; }
 
 bool valid_blk_quant(int blk) { return blk == 16 || blk == 32 || blk == 64 || blk == 128; }
-bool valid_blk_attn(int blk) { return blk == 32 || blk == 64 || blk == 128; }
-bool valid_blkk_attn(int blk) { return blk == 16 || valid_blk_attn(blk); }
+bool valid_blk_attn(int blk) { return blk == 16 || blk == 32 || blk == 64 || blk == 128; }
+bool valid_blkk_attn(int blk) { return valid_blk_attn(blk); }
 int ilog2(int x) { int r = 0; while ((1 << r) < x) r++; return r; }
 
 int check_common(int B, int H, int L, int D, int dtype) {
@@ -210,7 +210,7 @@ int attn_impl(const int8_t* q, const int8_t* k, const void* v_panels, const floa
   if (Skv < 0) return fail(SAGE_EINVAL, "negative kv length");
   if (pv_mode != SAGE_PV_FP16 && pv_mode != SAGE_PV_FP8) return fail(SAGE_EINVAL, "pv_mode %d unknown", pv_mode);
   if (!valid_blk_attn(blkq) || !valid_blkk_attn(blkk))
-    return fail(SAGE_ENOTIMPL, "attention needs Q scale blocks of 32/64/128 rows and K scale blocks of 16/32/64/128 rows (got %d/%d)", blkq, blkk);
+    return fail(SAGE_ENOTIMPL, "attention needs Q and K scale blocks of 16, 32, 64 or 128 rows (got %d/%d)", blkq, blkk);
   if (blkk == 16 && mask.ptr) return fail(SAGE_ENOTIMPL, "K scale blocks of 16 rows cannot be combined with an explicit mask");
   if (B == 0 || Hq == 0 || Sq == 0) return SAGE_OK;
   if (!k || !v_panels || !k_scale || !out) return fail(SAGE_EINVAL, "null tensor pointer");
@@ -366,7 +366,7 @@ int sage_sageattn_masked(const void* q, const void* k, const void* v, void* out,
   if (int rc = check_common(B, Hq, Sq, D, dtype)) return rc;
   if (Hkv <= 0 || Hq % Hkv) return fail(SAGE_EINVAL, "query heads (%d) must be divisible by KV heads (%d)", Hq, Hkv);
   if (!valid_blk_attn(blkq) || !valid_blkk_attn(blkk))
-    return fail(SAGE_ENOTIMPL, "Q scale blocks must be 32/64/128 rows and K scale blocks 16/32/64/128 rows (got %d/%d)", blkq, blkk);
+    return fail(SAGE_ENOTIMPL, "Q and K scale blocks must be 16, 32, 64 or 128 rows (got %d/%d)", blkq, blkk);
   if (pv_mode != SAGE_PV_FP16 && pv_mode != SAGE_PV_FP8) return fail(SAGE_EINVAL, "pv_mode %d unknown", pv_mode);
   const int varlen = cu_seqlens_q != nullptr;
   if (varlen && !cu_seqlens_k) return fail(SAGE_EINVAL, "packed mode needs cu_seqlens_k");

@@ -273,11 +273,11 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
     const int8_t* qp = a.q + qoff + (int64_t)min(my_row, Lq - 1) * a.q_sn + 16 * h;
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) qreg[ks] = *reinterpret_cast<const v4i*>(qp + 32 * ks);
-    qscale = qsp[min(row0, Lq - 1) >> a.blkq_shift];
+    qscale = qsp[min(my_row, Lq - 1) >> a.blkq_shift];   // per lane: scale blocks may be smaller than a wavefront's 32 rows
   } else {
     // Quantise this wavefront's 32 rows here, exactly as quant_int8_kernel would
     // (quant_per_block.py:38-46): x32 = fp32(x) * mult, scale = max|x32| / 127 over the scale block
-    // (32, 64 or 128 rows = 1, 2 or 4 wavefronts), q = trunc(x32 / scale + 0.5 sgn).  Rows past the
+    // (16 rows = half a wavefront; 32, 64 or 128 rows = 1, 2 or 4 wavefronts), q = trunc(x32 / scale + 0.5 sgn).  Rows past the
     // end repeat the last row, which belongs to the same (last) scale block or to none.
 #pragma clang fp contract(off)
     __shared__ float q_block_amax[NW];
@@ -313,7 +313,10 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
         amax = fmaxf(amax, fabsf(x[ks][i]));
       }
     }
-    amax = wave_max(amax);
+    // Scale blocks of 16 rows: the lanes of a DPP row hold 16 consecutive query rows (one column half each),
+    // the other column half sits 32 lanes away.  Larger blocks span the wavefront (and its neighbours, below).
+    if (a.blkq == 16) amax = xchg32_max(row16_max(amax));
+    else amax = wave_max(amax);
     SAGE_T(2, amax);   // the raw Q rows have arrived
     const int wpb = a.blkq >> 5;   // wavefronts per scale block
     if (wpb > 1) {

@@ -99,11 +99,16 @@ __device__ inline float dpp_f(float x) {
   return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, x), __builtin_bit_cast(int, x),
                                                               CTRL, 0xf, 0xf, false));
 }
-__device__ inline float wave_max(float x) {
+// Maximum over the 16 lanes of a DPP row (lanes 16r .. 16r+15), in every lane of the row.
+__device__ inline float row16_max(float x) {
   x = fmaxf(x, dpp_f<0xB1>(x));   // quad_perm [1,0,3,2]
   x = fmaxf(x, dpp_f<0x4E>(x));   // quad_perm [2,3,0,1]
   x = fmaxf(x, dpp_f<0x141>(x));  // row_half_mirror
   x = fmaxf(x, dpp_f<0x140>(x));  // row_mirror
+  return x;
+}
+__device__ inline float wave_max(float x) {
+  x = row16_max(x);
   float a = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), 0));
   float b = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), 16));
   float c = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), 32));

@@ -233,8 +233,8 @@ def forward(q, k, v, q_scale, k_scale, tensor_layout="HND", attn_mask=None, outp
         raise ValueError("query heads must be divisible by KV heads")
     if D not in (64, 128):
         raise NotImplementedError("head_dim must be 64 or 128")
-    if BLKQ not in (32, 64, 128) or BLKK not in (16, 32, 64, 128):
-        raise NotImplementedError("the attention kernel needs Q scale blocks of 32/64/128 and K scale blocks of 16/32/64/128 rows")
+    if BLKQ not in (16, 32, 64, 128) or BLKK not in (16, 32, 64, 128):
+        raise NotImplementedError("the attention kernel needs Q and K scale blocks of 16, 32, 64 or 128 rows")
     exp_q = (B, Hq, (Sq + BLKQ - 1) // BLKQ)
     exp_k = (B, Hkv, (Skv + BLKK - 1) // BLKK)
     if tuple(q_scale.shape) != exp_q:
@@ -290,8 +290,8 @@ def forward_fused_q(q, k, v, k_scale, tensor_layout="HND", sm_scale=None, output
         raise ValueError("query heads must be divisible by KV heads")
     if D not in (64, 128):
         raise NotImplementedError("head_dim must be 64 or 128")
-    if BLKQ not in (32, 64, 128) or BLKK not in (16, 32, 64, 128):
-        raise NotImplementedError("the fused-Q kernel needs Q scale blocks of 32/64/128 and K scale blocks of 16/32/64/128 rows")
+    if BLKQ not in (16, 32, 64, 128) or BLKK not in (16, 32, 64, 128):
+        raise NotImplementedError("the fused-Q kernel needs Q and K scale blocks of 16, 32, 64 or 128 rows")
     if tuple(k_scale.shape) != (B, Hkv, (Skv + BLKK - 1) // BLKK):
         raise ValueError(f"k_scale has shape {tuple(k_scale.shape)}, expected {(B, Hkv, (Skv + BLKK - 1) // BLKK)}")
     pv = _pv(pv_mode)
@@ -360,8 +360,8 @@ def sageattn(q, k, v, tensor_layout="HND", is_causal=False, sm_scale=None, smoot
         raise ValueError("query heads must be divisible by KV heads")
     if D not in (64, 128):
         raise NotImplementedError("head_dim must be 64 or 128")
-    if BLKQ not in (32, 64, 128) or BLKK not in (16, 32, 64, 128):
-        raise NotImplementedError("the attention kernel needs Q scale blocks of 32/64/128 and K scale blocks of 16/32/64/128 rows")
+    if BLKQ not in (16, 32, 64, 128) or BLKK not in (16, 32, 64, 128):
+        raise NotImplementedError("the attention kernel needs Q and K scale blocks of 16, 32, 64 or 128 rows")
     pv = _pv(pv_mode)
     out = torch.empty(q.shape, device=q.device, dtype=q.dtype)
     _, _, _, _, osb, osh, osn = _layout(out, tensor_layout)
@@ -426,8 +426,8 @@ def sageattn_varlen(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqle
         raise ValueError("query heads must be divisible by KV heads")
     if D not in (64, 128):
         raise NotImplementedError("head_dim must be 64 or 128")
-    if BLKQ not in (32, 64, 128) or BLKK not in (16, 32, 64, 128):
-        raise NotImplementedError("the attention kernel needs Q scale blocks of 32/64/128 and K scale blocks of 16/32/64/128 rows")
+    if BLKQ not in (16, 32, 64, 128) or BLKK not in (16, 32, 64, 128):
+        raise NotImplementedError("the attention kernel needs Q and K scale blocks of 16, 32, 64 or 128 rows")
     nseq = cu_seqlens_q.numel() - 1
     pv = _pv(pv_mode)
     out = torch.empty_like(q)

@@ -131,7 +131,7 @@ int sage_varlen_plan(const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k, i
  *   accumulation, O /= l, optional LSE2 = log2(l) + m  (lse[(b*Hq+h)*Sq + i], fp32).
  * plus causal masking (key j visible to query i iff j <= i) with block skipping, and packed
  * variable-length batches.  kvh = qh / (Hq/Hkv) (sageattention_triton.py:61).
- * q_scale/k_scale: as written by sage_quant_int8 with blkq in {32, 64, 128}, blkk in {16, 32, 64, 128}
+ * q_scale/k_scale: as written by sage_quant_int8 with blkq and blkk in {16, 32, 64, 128}
  * (16: the K granularity of the external recipe (128, 16), sage_attention_benchmark_compare.py:93).
  * v_panels/v_scale: as written by sage_prep_v (v_scale NULL for SAGE_PV_FP16).
  * out: fp16/bf16 (out_dtype) addressed with (o_sb,o_sh,o_sn), base and strides multiples of 16 bytes (rows are

@@ -78,7 +78,7 @@ def test_attn_argument_errors(sage_lib):
     assert call(Hq=3) == _cabi.SAGE_EINVAL          # heads not divisible
     assert call(D=32) == _cabi.SAGE_ENOTIMPL
     assert call(blkk=8) == _cabi.SAGE_ENOTIMPL       # K scale blocks: 16, 32, 64 or 128 rows
-    assert call(blkq=16) == _cabi.SAGE_ENOTIMPL      # Q scale blocks: 32, 64 or 128 rows
+    assert call(blkq=8) == _cabi.SAGE_ENOTIMPL       # Q scale blocks: 16, 32, 64 or 128 rows
     assert call(pv=1) == _cabi.SAGE_EINVAL           # fp8 needs v_scale
     assert call(pv=5) == _cabi.SAGE_EINVAL
 

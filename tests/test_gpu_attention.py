@@ -254,7 +254,30 @@ def test_sageattn_with_the_128_16_recipe_against_fp32_sdpa():
     ref = oa.sdpa_fp32(q, k, v, "NHD", True)
     assert oa.metrics(out.cpu().float(), ref)["cosine"] >= 0.999
     with pytest.raises(NotImplementedError):
-        sa.sageattn(q.to(DEV), k.to(DEV), v.to(DEV), tensor_layout="NHD", BLKQ=16, BLKK=16)
+        sa.sageattn(q.to(DEV), k.to(DEV), v.to(DEV), tensor_layout="NHD", BLKQ=8, BLKK=16)
+
+
+@pytest.mark.parametrize("pv", ["fp16", "fp8"])
+@pytest.mark.parametrize("causal", [False, True])
+def test_q_scale_blocks_of_16_rows(pv, causal):
+    """Q scale blocks of half a wavefront (16 rows): bit-exact INT8 operands, `forward` against the formula, and
+    the fused-Q kernels (sageattn, forward_fused_q) bit-identical to quantise-then-forward."""
+    g = torch.Generator().manual_seed(160 + int(causal))
+    q = randn("HND", 2, 4, 333, 128, torch.bfloat16, g)
+    k = randn("HND", 2, 2, 333, 128, torch.bfloat16, g)
+    v = randn("HND", 2, 2, 333, 128, torch.bfloat16, g)
+    qd, kd, vd = q.to(DEV), k.to(DEV), v.to(DEV)
+    qi, qs, ki, ks = sa.per_block_int8(qd, kd, BLKQ=16, BLKK=32)
+    rqi, rqs, rki, rks = oq.per_block_int8(q, k, BLKQ=16, BLKK=32)
+    assert torch.equal(qi.cpu(), rqi) and torch.equal(qs.cpu(), rqs) and tuple(qs.shape) == (2, 4, 21)
+    out, _ = sa.forward(qi, ki, vd, qs, ks, output_dtype=torch.bfloat16, BLKQ=16, BLKK=32, is_causal=causal, pv_mode=pv)
+    ref, _ = oa.sage_reference(qi.cpu(), ki.cpu(), v, qs.cpu(), ks.cpu(), "HND", 16, 32, is_causal=causal)
+    m = oa.metrics(out.cpu().float(), ref)
+    assert m["finite"] and (m["rel_rmse"] < 6e-3 if pv == "fp16" else m["cosine"] >= 0.999), m
+    fused, _ = sa.forward_fused_q(qd, ki, vd, ks, BLKQ=16, BLKK=32, is_causal=causal, pv_mode=pv)
+    assert torch.equal(fused, out)
+    one = sa.sageattn(qd, kd, vd, is_causal=causal, smooth_k=False, pv_mode=pv, BLKQ=16, BLKK=32)
+    assert torch.equal(one, out)
 
 
 @pytest.mark.parametrize("layout", ["HND", "NHD"])

@@ -20,7 +20,7 @@ LENGTHS = [1, 7, 31, 64, 100, 128, 129, 255, 256, 257, 300, 511, 513, 700, 1025]
 def _draw(rng):
     c = dict(D=rng.choice([64, 128]), dtype=rng.choice([torch.float16, torch.bfloat16]), layout=rng.choice(["HND", "NHD"]),
              Hkv=rng.choice([1, 2, 3, 8]), G=rng.choice([1, 1, 2, 4]), B=rng.choice([1, 1, 2, 3]), S=rng.choice(LENGTHS),
-             causal=rng.random() < 0.5, pv=rng.choice(["fp16", "fp8"]), blkq=rng.choice([32, 64, 128]),
+             causal=rng.random() < 0.5, pv=rng.choice(["fp16", "fp8"]), blkq=rng.choice([16, 32, 64, 128]),
              blkk=rng.choice([16, 32, 64, 128]), smooth=rng.random() < 0.7, lse=rng.random() < 0.3, seed=rng.randrange(1 << 30))
     c["Skv"] = c["S"] if (c["causal"] or rng.random() < 0.5) else rng.choice([1, 5, 64, 130, 260, 777])
     return c

@@ -91,7 +91,7 @@ def _draw_packed(rng):
     hkv = rng.choice([1, 2, 8])
     return dict(D=rng.choice([64, 128]), dtype=rng.choice([torch.float16, torch.bfloat16]), Hkv=hkv, Hq=hkv * rng.choice([1, 2, 4]),
                 lens=[rng.choice(lens_pool) for _ in range(rng.choice([1, 2, 3, 6, 9]))], causal=rng.random() < 0.5,
-                pv=rng.choice(["fp16", "fp8"]), blkq=rng.choice([32, 64, 128]), blkk=rng.choice([32, 64, 128]),
+                pv=rng.choice(["fp16", "fp8"]), blkq=rng.choice([16, 32, 64, 128]), blkk=rng.choice([32, 64, 128]),
                 smooth=rng.random() < 0.7, seed=rng.randrange(1 << 30))
 
 
