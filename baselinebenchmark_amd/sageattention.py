@@ -406,10 +406,13 @@ def _check_cu(name, cu, device):
 
 @torch.no_grad()
 def sageattn_varlen(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, is_causal=False, sm_scale=None,
-                    smooth_k=True, pv_mode="fp16", BLKQ=128, BLKK=64):
+                    smooth_k=True, pv_mode="fp16", BLKQ=128, BLKK=64, return_lse=False):
     """Packed variable-length attention: q [Tq, Hq, D], k/v [Tk, Hkv, D], cu_seqlens int32 [nseq+1]
     on the device.  Quantisation blocks and the K mean restart at every sequence; the (sequence,
-    q-tile) work list is built and cost-ordered on the device, so no host synchronisation happens."""
+    q-tile) work list is built and cost-ordered on the device, so no host synchronisation happens.
+    With ``return_lse=True`` returns ``(out, lse)``, lse [Hq, Tq] float32: the natural-log log-sum-exp of
+    ``sm_scale * q k^T`` (causal-masked if asked) of every packed row over its own sequence, for the original k
+    (what K smoothing removes is added back) -- the quantity a split-KV or ring merge needs."""
     for name, t in (("q", q), ("k", k), ("v", v)):
         _check_packed(name, t)
     _check_cu("cu_seqlens_q", cu_seqlens_q, q.device)
@@ -431,16 +434,19 @@ def sageattn_varlen(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqle
     nseq = cu_seqlens_q.numel() - 1
     pv = _pv(pv_mode)
     out = torch.empty_like(q)
+    lse = torch.empty((Hq, Tq), device=q.device, dtype=torch.float32) if return_lse else None
     ws_bytes = lib().sage_sageattn_workspace_bytes(nseq, Hq, Hkv, int(max_seqlen_q), int(max_seqlen_k), D, BLKQ, BLKK, pv,
                                                    Tq, Tk, 1)
     ws = torch.empty(max(ws_bytes, 256), device=q.device, dtype=torch.uint8)
-    check(lib().sage_sageattn(_ptr(q), _ptr(k), _ptr(v), _ptr(out), None, _ptr(ws), ws_bytes,
+    check(lib().sage_sageattn(_ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _ptr(ws), ws_bytes,
                               nseq, Hq, Hkv, int(max_seqlen_q), int(max_seqlen_k), D,
                               0, q.stride(1), q.stride(0), 0, k.stride(1), k.stride(0), 0, v.stride(1), v.stride(0),
                               0, out.stride(1), out.stride(0),
                               _dt(q.dtype), BLKQ, BLKK, float(D ** -0.5 if sm_scale is None else sm_scale),
                               int(bool(is_causal)), int(bool(smooth_k)), pv,
                               _ptr(cu_seqlens_q), _ptr(cu_seqlens_k), Tq, Tk, _stream(q)))
+    if return_lse:
+        return out, lse * 0.6931471805599453
     return out
 
 

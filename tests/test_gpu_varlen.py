@@ -108,3 +108,26 @@ def test_random_packed_batches_match_sdpa_and_the_fixed_length_call(c):
         assert m["finite"] and m["cosine"] >= 0.998, (i, c["lens"][i], m)
         one = sa.sageattn(qd[a:b].unsqueeze(0), kd[a:b].unsqueeze(0), vd[a:b].unsqueeze(0), tensor_layout="NHD", **kw)
         assert torch.equal(one[0], out[a:b]), (i, c["lens"][i])
+
+
+@pytest.mark.parametrize("smooth", [False, True])
+@pytest.mark.parametrize("causal", [False, True])
+def test_varlen_lse_is_the_per_sequence_logsumexp(smooth, causal):
+    lens = [257, 1, 600, 130]
+    Hq, Hkv, D = 4, 2, 128
+    q, k, v, cu = _packed(lens, Hq, Hkv, D, torch.float16, 21)
+    out, lse = sa.sageattn_varlen(q.to(DEV), k.to(DEV), v.to(DEV), cu.to(DEV), cu.to(DEV), max(lens), max(lens),
+                                  is_causal=causal, smooth_k=smooth, pv_mode="fp16", return_lse=True)
+    plain = sa.sageattn_varlen(q.to(DEV), k.to(DEV), v.to(DEV), cu.to(DEV), cu.to(DEV), max(lens), max(lens),
+                               is_causal=causal, smooth_k=smooth, pv_mode="fp16")
+    assert tuple(lse.shape) == (Hq, int(cu[-1])) and lse.dtype == torch.float32
+    assert oa.metrics(out.cpu().float(), plain.cpu().float())["cosine"] >= 0.99999      # same attention, with or without LSE
+    for i, L in enumerate(lens):
+        a, b = int(cu[i]), int(cu[i + 1])
+        qs = q[a:b].double().transpose(0, 1)                                  # [Hq, L, D]
+        ks = k[a:b].double().transpose(0, 1).repeat_interleave(Hq // Hkv, dim=0)
+        logits = torch.matmul(qs, ks.transpose(-1, -2)) * D ** -0.5
+        if causal:
+            logits = logits.masked_fill(~torch.ones(L, L, dtype=torch.bool).tril(), -float("inf"))
+        ref = torch.logsumexp(logits, dim=-1)
+        assert (lse[:, a:b].cpu().double() - ref).abs().max().item() < 6e-2, (i, L)     # INT8 noise on the logits
