@@ -21,7 +21,10 @@
 //     q_scale*k_scale and subtracts the running maximum.
 //   * The running maximum is only moved when it grows by more than kTau (lazy rescale); P is stored
 //     with a static 2^kPShift so that fp8's range [2^-9, 448] is used.
-//   * K/V tiles go global -> LDS directly (buffer_load ... lds, no registers), two slots each.
+//   * K/V tiles go global -> LDS directly (buffer_load ... lds, no registers): four slots per stream and
+//     requests two tile periods ahead for FP8 P.V, two slots and one period for FP16 P.V.  The raw q-tile of
+//     the variants that quantise their own Q and the V scales of the epilogue arrive the same way, and the
+//     output leaves through an LDS transposition as whole rows.
 //   * The wavefronts of a workgroup form two groups that run half a tile apart, two barriers per tile:
 //     while one group feeds the matrix pipe (P.V of its last tile, Q.K^T of its next) the other runs
 //     the softmax of the tile in between on the vector ALU.  Wavefronts w and w+4 share a SIMD and
