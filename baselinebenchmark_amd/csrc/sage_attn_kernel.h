@@ -44,6 +44,7 @@ constexpr float kBiasF = 12582912.0f;     // 1.5 * 2^23
 constexpr int kBiasBits = 0x4B400000;     // its bit pattern; int accumulators start here
 constexpr float kNegInf = -__builtin_inff();
 constexpr float kMInit = -1.0e30f;
+constexpr float kCodeBias = -0.3f;       // centres the linear-mantissa fp8 code of the probabilities (see softmax)
 
 template <int PV> struct PCfg;
 template <> struct PCfg<1> { static constexpr float tau = 3.0f, pshift = 5.0f; };   // fp8: p*32 <= 256 < 448
@@ -142,6 +143,14 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
   constexpr int CPR = D / 16;
   constexpr float TAU = PCfg<PV>::tau, PSHIFT = PCfg<PV>::pshift;
   constexpr int NSLOT = attn_tile_slots<PV, CAUSAL>(), LEAD = attn_tile_lead<PV, CAUSAL>();   // tiles are requested LEAD periods ahead
+  // FP8 P.V: the softmax denominator of O always comes from the matrix pipe (the sum of the very fp8 values that
+  // multiply V); MSUM additionally means that no fp32 sum is kept (no LSE wanted), and then the probabilities are
+  // coded without v_exp_f32 (FASTP, see softmax).
+  constexpr bool RSUM = PV == 1;
+  constexpr bool FASTP = PV == 1 && MSUM && MASK == 0;
+  // FP8 kernels take the row maximum in the vector phase (their softmax is short) and let the group that is in its
+  // vector phase issue the tile requests; FP16 kernels keep both in the matrix phase.
+  constexpr bool VECMAX = PV == 1;
 
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
@@ -225,40 +234,44 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
   auto vslot = [&](int j) { return smem + NSLOT * KBYTES + (j % NSLOT) * VBYTES; };
   // Per-lane byte offsets of this wavefront's pieces inside a tile are loop invariant; the tile index
   // only adds a uniform term.  Rows past the end of the sequence (last tile only) are clamped.
+  // Piece offsets are those of the lower wavefront of the SIMD pair (wl); dw selects which wavefront's pieces a
+  // request covers: dw_self for this wavefront's own (prologue), 0 and PARTNER_DW for both of the pair (main
+  // loop, where one wavefront issues for two).  Offsets added per request are therefore never negative.
+  constexpr int PARTNER_DW = 1 << GSH;
+  const int wl = w & ~PARTNER_DW, dw_self = w - wl;
   int koffv[KPIECES], voffv[VPIECES];
 #pragma unroll
   for (int i = 0; i < KPIECES; i++) {
-    const int sl = (i * NW + w) * 64 + lane, n = sl / CPR, cc = (sl % CPR) ^ kswz<D>(n);
+    const int sl = (i * NW + wl) * 64 + lane, n = sl / CPR, cc = (sl % CPR) ^ kswz<D>(n);
     koffv[i] = n * (int)a.k_sn + 16 * cc;
   }
 #pragma unroll
-  for (int i = 0; i < VPIECES; i++) voffv[i] = (i * NW + w) * 1024 + lane * 16;
+  for (int i = 0; i < VPIECES; i++) voffv[i] = (i * NW + wl) * 1024 + lane * 16;
   const int ktile_bytes = BN * (int)a.k_sn;
-  // dw: load the pieces of wavefront w + dw instead of this wavefront's own.  dw is a multiple of 4, so
-  // the rows move by a multiple of 16 and keep their swizzle: only the uniform offset changes.
+  // dw is a multiple of 4, so the rows move by a multiple of 16 and keep their swizzle: only the uniform offset changes.
   auto load_k = [&](int j, int dw) {
     uint8_t* dst = kslot(j) + dw * 1024;
     if (j * BN + BN <= Lk) {
       const int uo = j * ktile_bytes + dw * (64 / CPR) * (int)a.k_sn;
 #pragma unroll
-      for (int i = 0; i < KPIECES; i++) dma16(krsrc, koffv[i], uo, dst + (i * NW + w) * 1024);
+      for (int i = 0; i < KPIECES; i++) dma16(krsrc, koffv[i], uo, dst + (i * NW + wl) * 1024);
     } else {
 #pragma unroll
       for (int i = 0; i < KPIECES; i++) {
-        const int sl = (i * NW + w + dw) * 64 + lane, n = sl / CPR, cc = (sl % CPR) ^ kswz<D>(n);
-        dma16(krsrc, min(j * BN + n, Lk - 1) * (int)a.k_sn + 16 * cc, 0, dst + (i * NW + w) * 1024);
+        const int sl = (i * NW + wl + dw) * 64 + lane, n = sl / CPR, cc = (sl % CPR) ^ kswz<D>(n);
+        dma16(krsrc, min(j * BN + n, Lk - 1) * (int)a.k_sn + 16 * cc, 0, dst + (i * NW + wl) * 1024);
       }
     }
   };
   auto load_v = [&](int j, int dw) {
     uint8_t* dst = vslot(j) + dw * 1024;
 #pragma unroll
-    for (int i = 0; i < VPIECES; i++) dma16(vrsrc, voffv[i], j * VBYTES + dw * 1024, dst + (i * NW + w) * 1024);
+    for (int i = 0; i < VPIECES; i++) dma16(vrsrc, voffv[i], j * VBYTES + dw * 1024, dst + (i * NW + wl) * 1024);
   };
 
   // The first K tile is requested before anything else waits on memory, and the per-channel V scales
   // of the epilogue come along (4 bytes per lane, D / 64 wavefronts).
-  if (ntiles > 0) load_k(0, 0);
+  if (ntiles > 0) load_k(0, dw_self);
   float* vs_lds = reinterpret_cast<float*>(smem + attn_tile_lds_bytes<D, NW, BN, PV, CAUSAL, QF>());
   if constexpr (PV == 1) {
     if (w < D / 64) {
@@ -349,7 +362,7 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
 
 
   // With two periods of lead the second K tile follows as soon as the raw Q rows are out of the way.
-  if (LEAD == 2 && ntiles > 1) load_k(1, 0);
+  if (LEAD == 2 && ntiles > 1) load_k(1, dw_self);
 
   v16i bias;
 #pragma unroll
@@ -362,12 +375,11 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
 #pragma unroll
     for (int i = 0; i < 16; i++) o[dt][i] = 0.f;
   float m_used = kMInit, lsum = 0.f;
-  // MSUM (FP8 mode when no LSE is requested): the row sums come out of the matrix pipe too.  A V^T operand of all ones (fp8 1.0 = 0x38)
+  // FP8 P.V: the row sums come out of the matrix pipe too.  A V^T operand of all ones (fp8 1.0 = 0x38)
   // makes every row of one extra 32x32 output tile equal to sum_n P[n][m], i.e. the softmax
-  // denominator of query row m -- of the very fp8 values that multiply V.  That removes one VALU add
-  // per score (the VALU, not the MFMA pipe, is the busier unit of this kernel).  The sum of rounded
+  // denominator of query row m -- of the very fp8 values that multiply V.  The sum of rounded
   // values is the right denominator for O but costs LSE accuracy on rows with few keys, so kernels
-  // that return LSE keep the fp32 VALU sum.
+  // that return LSE (MSUM false) also keep the fp32 sum of the unrounded values on the vector ALU, for LSE alone.
   v16f osum;
 #pragma unroll
   for (int i = 0; i < 16; i++) osum[i] = 0.f;
@@ -489,7 +501,7 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
       const float m_new = fmaxf(m_used, mall);
       const float alpha = __builtin_amdgcn_exp2f(m_used - m_new);
       lsum *= alpha;
-      if constexpr (MSUM) {
+      if constexpr (RSUM) {
 #pragma unroll
         for (int i = 0; i < 16; i++) osum[i] *= alpha;
       }
@@ -500,7 +512,37 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
       m_used = m_new;
     }
     // P = exp2(S - m) * 2^PSHIFT, packed straight into the B operand of the second MFMA
-    if constexpr (PV == 1) {
+    if constexpr (FASTP) {
+      // The byte of an e4m3 number, read as an integer, is 8*(exponent + 7) + mantissa: piecewise linear in
+      // log2 of the value.  So u8(round(8*t + 56)) is the fp8 code of a number within a mantissa step of
+      // 2^t, with the mantissa interpolated linearly between powers of two instead of exponentially
+      // (kCodeBias centres the error of that, at most a third of a code step).  One v_fma_f32 and one
+      // v_cvt_pk_u8_f32 (round to nearest even, saturating at 0: masked scores are -inf and give +0) per
+      // score replace v_fma_f32 + v_exp_f32 + half a v_cvt_pk_fp8_f32: the vector ALU is the busier pipe.
+      // t <= PSHIFT + TAU = 8, so the code stays <= 120 (= 256.0), below 0x7f.  The row sums of these very
+      // codes come from the matrix pipe, so numerator and denominator of O see the same values.
+      const float k0 = 8.0f * (PSHIFT - m_used) + (56.0f + kCodeBias);
+#pragma unroll
+      for (int nt = 0; nt < NT; nt++) {
+        float c[KSUB], mul[KSUB];
+#pragma unroll
+        for (int sub = 0; sub < KSUB; sub++) {
+          mul[sub] = 8.0f * sc[nt * KSUB + sub];
+          c[sub] = __builtin_fmaf(-kBiasF, mul[sub], k0);
+        }
+        float t8[16];
+#pragma unroll
+        for (int r = 0; r < 16; r++) t8[r] = __builtin_fmaf(as_f(acc[nt][r]), mul[KSUB == 2 ? r / 8 : 0], c[KSUB == 2 ? r / 8 : 0]);
+#pragma unroll
+        for (int q4 = 0; q4 < 4; q4++) {
+          // all four bytes get written, so the 'old' operand of the first insertion is a don't-care
+          unsigned d = (unsigned)acc[0][4 * nt + q4];
+#pragma unroll
+          for (int e = 0; e < 4; e++) d = __builtin_amdgcn_cvt_pk_u8_f32(t8[4 * q4 + e], e, d);
+          acc[0][4 * nt + q4] = (int)d;
+        }
+      }
+    } else if constexpr (PV == 1) {
 #pragma unroll
       for (int nt = 0; nt < NT; nt++) {
         float c[KSUB], mul[KSUB];
@@ -513,7 +555,7 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
 #pragma unroll
         for (int r = 0; r < 16; r++) {
           p[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(as_f(acc[nt][r]), mul[KSUB == 2 ? r / 8 : 0], c[KSUB == 2 ? r / 8 : 0]));
-          if constexpr (!MSUM) lsum += p[r];
+          if constexpr (!MSUM) lsum += p[r];   // the unrounded sum, for LSE only
         }
 #pragma unroll
         for (int q4 = 0; q4 < 4; q4++) {
@@ -571,7 +613,7 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
         v8i pb;
 #pragma unroll
         for (int e = 0; e < 8; e++) pb[e] = acc[0][8 * kk + e];
-        if constexpr (MSUM) {
+        if constexpr (RSUM) {
           if (dt == 0) osum = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ones, pb, osum, 0, 0, 0, 0, 0, 0);
         }
         o[dt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vf[i], pb, o[dt], 0, 0, 0, 0, 0, 0);
@@ -579,7 +621,7 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
       __builtin_amdgcn_sched_group_barrier(0x100, 2 * VPF, 0);
 #pragma unroll
       for (int i = 0; i < NV; i++) {
-        if (MSUM && i % DTN == 0) __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        if (RSUM && i % DTN == 0) __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
         if (i + VPF < NV) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
       }
@@ -647,20 +689,54 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
 #endif
     };
     const int first_in_flight = (LEAD == 2 && ntiles > 1) ? KPIECES : 0;   // the second K tile, requested in the prologue
-    if (grp == 0) {
-      // The even phase is as long as group 1's softmax, which must not start late: all tile loads of the
-      // period are issued here, by the group whose matrix phase has slack, after its P.V.  Period j requests
-      // K(j+LEAD) and V(j+LEAD-1), LEAD periods before their first use (a tile that has to come from HBM takes
-      // longer than one period), into the slots whose last readers finished a barrier ago; with LEAD = 2,
-      // V(0) goes first in period 0 and the requests of the last period may still be in flight at a barrier.
-      constexpr int PARTNER = 1 << GSH;
-      constexpr int NK = 2 * KPIECES, NV = 2 * VPIECES;   // requests per K / V tile of a group-0 wavefront
+    constexpr int PARTNER = PARTNER_DW;
+    constexpr int NK = 2 * KPIECES, NV = 2 * VPIECES;   // requests per K / V tile of the wavefront that issues for its SIMD pair
+    // Tile requests of period j, issued by one wavefront for both wavefronts of its SIMD pair: K(j+LEAD) and
+    // V(j+LEAD-1), LEAD periods before their first use (a tile that has to come from HBM takes longer than one
+    // period), into the slots whose last readers finished a barrier ago; with LEAD = 2, V(0) goes first in
+    // period 0 and the requests of the last period may still be in flight at a barrier.
+    auto request_tiles = [&](int j) {
+      if (LEAD == 2 && j == 0) { load_v(0, 0); load_v(0, PARTNER); }
+      if (j + LEAD < ntiles) { load_k(j + LEAD, 0); load_k(j + LEAD, PARTNER); }
+      if (j + LEAD - 1 < ntiles) { load_v(j + LEAD - 1, 0); load_v(j + LEAD - 1, PARTNER); }
+    };
+    auto issuer_in_flight = [&](int j) {
+      return j == 0 ? first_in_flight : LEAD == 1 ? 0 : (j + 1 < ntiles ? NK : 0) + (j < ntiles ? NV : 0);
+    };
+#ifdef SAGE_NO_ODD_BARRIER
+    auto odd_barrier = [&]() {};
+#else
+    auto odd_barrier = [&]() { lds_barrier(); };
+#endif
+    if constexpr (VECMAX) {
+      // FP8 P.V: the matrix phase is nothing but MFMAs and their LDS reads (P.V of the previous tile, Q.K^T of the
+      // next); the row maximum, the probabilities and the tile requests all belong to the vector phase, which
+      // is the shorter one.  Group 1, whose vector phase is the even one, issues the requests.
+      if (grp == 0) {
+        for (int j = 0; j <= ntiles; j++) {
+          even_barrier(j, j == 0 ? first_in_flight : 0);
+          if (j >= 1 && j - 1 < wnt) pv(j - 1);
+          if (j < wnt) qk(j);
+          odd_barrier();
+          if (j < wnt) { rowmax(j); softmax(j); }
+        }
+      } else {
+        for (int j = 0; j <= ntiles; j++) {
+          even_barrier(j, issuer_in_flight(j));
+          if (j >= 1 && j - 1 < wnt) { rowmax(j - 1); softmax(j - 1); }
+          request_tiles(j);
+          odd_barrier();
+          if (j >= 1 && j - 1 < wnt) pv(j - 1);
+          if (j < wnt) qk(j);
+        }
+      }
+    } else if (grp == 0) {
+      // FP16 P.V.  The even phase is as long as group 1's softmax, which must not start late: all tile loads of
+      // the period are issued here, by the group whose matrix phase has slack, after its P.V.
       for (int j = 0; j <= ntiles; j++) {
-        even_barrier(j, j == 0 ? first_in_flight : LEAD == 1 ? 0 : (j + 1 < ntiles ? NK : 0) + (j < ntiles ? NV : 0));
+        even_barrier(j, issuer_in_flight(j));
         if (j >= 1 && j - 1 < wnt) pv(j - 1);
-        if (LEAD == 2 && j == 0) { load_v(0, 0); load_v(0, PARTNER); }
-        if (j + LEAD < ntiles) { load_k(j + LEAD, 0); load_k(j + LEAD, PARTNER); }
-        if (j + LEAD - 1 < ntiles) { load_v(j + LEAD - 1, 0); load_v(j + LEAD - 1, PARTNER); }
+        request_tiles(j);
         if (j < wnt) { qk(j); rowmax(j); }
         lds_barrier();
         if (j < wnt) softmax(j);
@@ -677,9 +753,12 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
 
   SAGE_T(5, lsum);   // main loop done
   // ---- epilogue: O = O^T / l (* v_scale), LSE2 = m + log2(l) ----
-  if constexpr (MSUM) lsum = osum[0];   // already the full row sum (the MFMA contracts over both lane halves)
+  // The denominator of O: FP8 kernels take the matrix pipe's sum of the rounded probabilities (already the full row
+  // sum: the MFMA contracts over both lane halves); the fp32 sum of the unrounded ones serves LSE only.
+  if constexpr (MSUM) lsum = osum[0];
   else lsum = xchg32_sum(lsum);
-  const float inv = lsum > 0.f ? 1.0f / lsum : 0.f;
+  const float den = RSUM ? osum[0] : lsum;
+  const float inv = den > 0.f ? 1.0f / den : 0.f;
   if (my_row < Lq) {
     if (a.lse && h == 0) {
       // lse_offset: what K smoothing removed from every logit of this row (q . k_mean, base-2 units)

@@ -207,7 +207,7 @@ def test_long_sequence_properties_full_size_head():
     out3, _ = sa.forward(qi, ki, vg, qs, ks, output_dtype=torch.bfloat16, BLKQ=64, BLKK=128, is_causal=True, pv_mode="fp8")
     out4, _ = sa.forward(qi, ki, vg * 2, qs, ks, output_dtype=torch.bfloat16, BLKQ=64, BLKK=128, is_causal=True, pv_mode="fp8")
     assert torch.equal(out4.cpu().float(), out3.cpu().float() * 2)
-    assert oa.metrics(out3.cpu().float(), o)["cosine"] >= 0.9995
+    assert oa.metrics(out3.cpu().float(), o)["cosine"] >= 0.999
 
 
 def test_lse_is_empty_unless_requested():
