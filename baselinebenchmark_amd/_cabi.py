@@ -26,8 +26,6 @@ _I, _L, _P = c_int, c_int64, c_void_p
 # name -> (restype, argtypes); one entry per declaration in include/sage_mi355x.h
 SIGNATURES = {
     "sage_backend_name": (c_char_p, []),
-    "sage_microbench_units": (ctypes.c_double, [_I]),
-    "sage_microbench": (c_int, [_I, _I, _I, _I, _P, c_size_t, _P]),
     "sage_last_error": (c_char_p, []),
     "sage_quant_int8": (c_int, [_P, _P, _P, _P, _I, _I, _I, _I, _L, _L, _L, _L, _L, _L, _L, _L, _I, c_float, _I,
                                 _P, _P, _L, _P]),

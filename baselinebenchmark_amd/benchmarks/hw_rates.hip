@@ -5,8 +5,8 @@
 //
 // One workgroup per compute unit, 1, 2 or 4 wavefronts per SIMD; the caller times the launch (the
 // in-kernel clock s_memtime does not advance at wall-clock rate when wavefronts share a SIMD).
-#include "sage_common.h"
-#include "../../include/sage_mi355x.h"
+#include "../csrc/sage_common.h"
+#include "hw_rates.h"
 
 namespace sage {
 namespace {
@@ -140,12 +140,12 @@ double sage_microbench_units(int kind) {
 }
 
 // Launches benchmark `kind` on `grid` workgroups of 4 * waves_per_simd wavefronts (waves_per_simd 1, 2 or 4), `iters`
-// iterations each.  `sink` receives one int per thread (grid * 1024 ints).  Returns 0 or a negative SAGE_E* code.
-int sage_microbench(int kind, int grid, int waves_per_simd, int iters, void* sink, size_t sink_bytes, sage_stream_t stream) {
+// iterations each.  `sink` receives one int per thread (grid * 1024 ints).  Returns 0 or a negative HWR_E* code.
+int sage_microbench(int kind, int grid, int waves_per_simd, int iters, void* sink, size_t sink_bytes, void* stream) {
   using namespace sage;
-  if (kind < 0 || kind >= MB_KINDS || grid <= 0 || grid > 65535 || iters <= 0 || !sink) return SAGE_EINVAL;
-  if (waves_per_simd != 1 && waves_per_simd != 2 && waves_per_simd != 4) return SAGE_EINVAL;
-  if (sink_bytes < (size_t)grid * 1024 * sizeof(int)) return SAGE_EWORKSPACE;
+  if (kind < 0 || kind >= MB_KINDS || grid <= 0 || grid > 65535 || iters <= 0 || !sink) return HWR_EINVAL;
+  if (waves_per_simd != 1 && waves_per_simd != 2 && waves_per_simd != 4) return HWR_EINVAL;
+  if (sink_bytes < (size_t)grid * 1024 * sizeof(int)) return HWR_ESIZE;
   int* out = (int*)sink;
   const int waves = 4 * waves_per_simd;
   hipStream_t st = (hipStream_t)stream;
@@ -161,7 +161,7 @@ int sage_microbench(int kind, int grid, int waves_per_simd, int iters, void* sin
     case MB_CVT_FP8: e = launch_mb<MB_CVT_FP8>(out, grid, waves, iters, st); break;
     default: e = launch_mb<MB_SOFTMAX_MIX>(out, grid, waves, iters, st); break;
   }
-  return e == hipSuccess ? SAGE_OK : SAGE_ELAUNCH;
+  return e == hipSuccess ? HWR_OK : HWR_ELAUNCH;
 }
 
 }  // extern "C"

@@ -14,7 +14,7 @@ from pathlib import Path
 
 CSRC = Path(__file__).resolve().parent / "csrc"
 LIB = CSRC / "libsage_mi355x.so"
-SOURCES = ["sage_quant.hip", "sage_attn.hip", "sage_attn_mask.hip", "sage_attn_qfuse.hip", "sage_microbench.hip", "sage_api.hip"]
+SOURCES = ["sage_quant.hip", "sage_attn.hip", "sage_attn_mask.hip", "sage_attn_qfuse.hip", "sage_api.hip"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     # correctly rounded fp32 divide (the INT8 quantiser's contract) and no packed-fp32 selection
@@ -44,12 +44,7 @@ def _compile(src: str, timing: bool = False) -> Path:
     return obj
 
 
-def build(verbose: bool = True, timing: bool = False) -> Path:
-    """Builds the library; ``timing=True`` builds the instrumented twin (``-DSAGE_TIMING=1``) next to it instead,
-    for ``python -m baselinebenchmark_amd.benchmarks.tile_timing``."""
-    lib = TIMING_LIB if timing else LIB
-    with ThreadPoolExecutor(max_workers=len(SOURCES)) as ex:
-        objs = list(ex.map(lambda src: _compile(src, timing), SOURCES))
+def _link(objs, lib: Path, verbose: bool) -> Path:
     cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", *map(str, objs), "-o", str(lib)]
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
@@ -59,5 +54,43 @@ def build(verbose: bool = True, timing: bool = False) -> Path:
     return lib
 
 
+def build(verbose: bool = True, timing: bool = False) -> Path:
+    """Builds the library; ``timing=True`` builds the instrumented twin (``-DSAGE_TIMING=1``) next to it instead,
+    for ``python -m baselinebenchmark_amd.benchmarks.tile_timing``."""
+    with ThreadPoolExecutor(max_workers=len(SOURCES)) as ex:
+        objs = list(ex.map(lambda src: _compile(src, timing), SOURCES))
+    return _link(objs, TIMING_LIB if timing else LIB, verbose)
+
+
+BENCH = Path(__file__).resolve().parent / "benchmarks"
+HWRATES_LIB = BENCH / "libsage_hwrates.so"      # hardware-rate micro-benchmarks (benchmarks/hw_rates.py)
+CABI_BENCH = BENCH / "sage_bench"               # C++ benchmark driver that calls the C ABI directly
+
+
+def build_tools(verbose: bool = True) -> list[Path]:
+    """Builds what the benchmark tools need and the drop-in library does not contain: the instrumented twin of the
+    library (tile_timing), the hardware-rate micro-benchmarks (hw_rates) and the C++ benchmark driver."""
+    out = [build(verbose, timing=True)]
+    obj = BENCH / "hw_rates.o"
+    res = subprocess.run([_hipcc(), *FLAGS, "-c", str(BENCH / "hw_rates.hip"), "-o", str(obj)], capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"hipcc failed for hw_rates.hip:\n{res.stderr}")
+    out.append(_link([obj], HWRATES_LIB, verbose))
+    src = BENCH / "sage_bench.cpp"
+    if src.exists():
+        cmd = [_hipcc(), "-O2", "-std=c++17", "-x", "hip", "--offload-arch=gfx950", str(src), "-I", str(CSRC.parent.parent / "include"),
+               "-L", str(CSRC), "-lsage_mi355x", f"-Wl,-rpath,{CSRC}", "-o", str(CABI_BENCH)]
+        res = subprocess.run(cmd, capture_output=True, text=True)
+        if res.returncode != 0:
+            raise RuntimeError(f"hipcc failed for sage_bench.cpp:\n{res.stderr}")
+        if verbose:
+            print(f"built {CABI_BENCH}")
+        out.append(CABI_BENCH)
+    return out
+
+
 if __name__ == "__main__":
-    build(timing="--timing" in sys.argv[1:])
+    if "--tools" in sys.argv[1:]:
+        build_tools()
+    else:
+        build(timing="--timing" in sys.argv[1:])

@@ -51,6 +51,10 @@ int check_stride16(const char* name, int64_t sb, int64_t sh, int64_t sn, int esz
 
 }  // namespace
 
+namespace sage {
+int set_error(int code, const char* msg) { return fail(code, "%s", msg); }
+}  // namespace sage
+
 extern "C" {
 
 const char* sage_backend_name(void) { return "mi355x_hip_int8_qk_fp8_fp16_pv"; }
@@ -213,7 +217,7 @@ int attn_impl(const int8_t* q, const int8_t* k, const void* v_panels, const floa
     return fail(SAGE_ENOTIMPL, "attention needs Q and K scale blocks of 16, 32, 64 or 128 rows (got %d/%d)", blkq, blkk);
   if (blkk == 16 && mask.ptr) return fail(SAGE_ENOTIMPL, "K scale blocks of 16 rows cannot be combined with an explicit mask");
   if (B == 0 || Hq == 0 || Sq == 0) return SAGE_OK;
-  if (!k || !v_panels || !k_scale || !out) return fail(SAGE_EINVAL, "null tensor pointer");
+  if (!out || (Skv > 0 && (!k || !v_panels || !k_scale))) return fail(SAGE_EINVAL, "null tensor pointer");
   if (!qraw.ptr && (!q || !q_scale)) return fail(SAGE_EINVAL, "null tensor pointer");
   if (qraw.ptr && mask.ptr) return fail(SAGE_ENOTIMPL, "fused Q quantisation: not with an explicit mask");
   if (pv_mode == SAGE_PV_FP8 && !v_scale) return fail(SAGE_EINVAL, "fp8 P.V needs v_scale");
@@ -386,8 +390,11 @@ int sage_sageattn_masked(const void* q, const void* k, const void* v, void* out,
   void* stat = ws + w.stat;
   int32_t* plan = varlen ? (int32_t*)(ws + w.plan) : nullptr;
   const size_t stat_bytes = w.plan - w.stat;
-  // the int8 copies are dense in the caller's layout order: reuse the input strides scaled to D
-  // (HND/NHD/packed inputs are dense, so their element strides are valid for an int8 tensor too)
+  // The int8 copies of q and k are the library's own tensors: they get dense strides of their own ([B,H,L,D] with
+  // whole rows contiguous, or packed [T,H,D]), whatever strides the caller's q and k have (views of a fused QKV
+  // buffer, sliced heads, ...), so that they always fit the workspace regions sized for B*H*L*D bytes.
+  const int64_t qi_sb = varlen ? 0 : (int64_t)Hq * Sq * D, qi_sh = varlen ? D : (int64_t)Sq * D, qi_sn = varlen ? (int64_t)Hq * D : D;
+  const int64_t ki_sb = varlen ? 0 : (int64_t)Hkv * Skv * D, ki_sh = varlen ? D : (int64_t)Skv * D, ki_sn = varlen ? (int64_t)Hkv * D : D;
   const int32_t *cu_qblk = nullptr, *cu_kblk = nullptr, *cu_panel = nullptr;
   if (varlen) {
     int rc = sage_varlen_plan(cu_seqlens_q, cu_seqlens_k, B, total_q, blkq, blkk, is_causal, plan,
@@ -396,12 +403,16 @@ int sage_sageattn_masked(const void* q, const void* k, const void* v, void* out,
     SagePlanLayout L = plan_layout(B, total_q);
     cu_qblk = plan + L.cu_qblk; cu_kblk = plan + L.cu_kblk; cu_panel = plan + L.cu_panel;
   }
-  int rc;
+  int rc = SAGE_OK;
+  // No keys at all (fixed-length mode): nothing to smooth, quantise or lay out; the attention kernel writes zeros
+  // and LSE = -inf without reading K, V or their scales.
+  const bool no_keys = !varlen && Skv == 0;
+  if (no_keys) smooth_k = 0;
   if (smooth_k) {
     rc = sage_k_mean(k, km, stat, stat_bytes, B, Hkv, Skv, D, k_sb, k_sh, k_sn, dtype, cu_seqlens_k, stream);
     if (rc) return rc;
   }
-  rc = sage_quant_int8(k, k_i8, k_scale, smooth_k ? km : nullptr, B, Hkv, Skv, D, k_sb, k_sh, k_sn, k_sb, k_sh, k_sn,
+  if (!no_keys) rc = sage_quant_int8(k, k_i8, k_scale, smooth_k ? km : nullptr, B, Hkv, Skv, D, k_sb, k_sh, k_sn, ki_sb, ki_sh, ki_sn,
                        (int64_t)Hkv * D, D, blkk, 1.0f, dtype, cu_seqlens_k, cu_kblk, w.ks_sh, stream);
   if (rc) return rc;
   // With K smoothing every logit of a query row loses q . k_mean; the softmax does not notice but the
@@ -418,13 +429,15 @@ int sage_sageattn_masked(const void* q, const void* k, const void* v, void* out,
   const float q_mult = (float)((sm_scale > 0 ? sm_scale : 1.0 / sqrt((double)D)) * 1.44269504);
   const bool fuse_q = !attn_mask && !lse_off;
   if (!fuse_q) {
-    rc = quant_impl(q, q_i8, q_scale, nullptr, B, Hq, Sq, D, q_sb, q_sh, q_sn, q_sb, q_sh, q_sn, 0, 0, blkq, q_mult, dtype,
+    rc = quant_impl(q, q_i8, q_scale, nullptr, B, Hq, Sq, D, q_sb, q_sh, q_sn, qi_sb, qi_sh, qi_sn, 0, 0, blkq, q_mult, dtype,
                     cu_seqlens_q, cu_qblk, w.qs_sh, dot, stream);
     if (rc) return rc;
   }
-  rc = sage_prep_v(v, panels, v_scale, stat, stat_bytes, B, Hkv, Skv, D, v_sb, v_sh, v_sn, dtype, pv_mode, cu_seqlens_k,
-                   cu_panel, w.panel_sh, stream);
-  if (rc) return rc;
+  if (!no_keys) {
+    rc = sage_prep_v(v, panels, v_scale, stat, stat_bytes, B, Hkv, Skv, D, v_sb, v_sh, v_sn, dtype, pv_mode, cu_seqlens_k,
+                     cu_panel, w.panel_sh, stream);
+    if (rc) return rc;
+  }
   QRawArg qr;
   if (fuse_q) { qr.ptr = q; qr.dtype = dtype; qr.mult = q_mult; }
   MaskArg m;
@@ -432,9 +445,11 @@ int sage_sageattn_masked(const void* q, const void* k, const void* v, void* out,
     // sageattn's additive mask is in natural-log units on top of sm_scale * q.k (test_sage_attention_mate.py:171-176)
     m.ptr = attn_mask; m.kind = mask_kind; m.sb = m_sb; m.sh = m_sh; m.sm = m_sm; m.sn = m_sn; m.mult = 1.44269504f;
   }
+  // the attention kernel reads either the caller's floating-point q (its strides) or the int8 copy (dense strides)
   return attn_impl(q_i8, k_i8, panels, q_scale, k_scale, pv_mode == SAGE_PV_FP8 ? v_scale : nullptr, out, lse, B, Hq, Hkv, Sq,
-                   Skv, D, q_sb, q_sh, q_sn, k_sb, k_sh, k_sn, o_sb, o_sh, o_sn, blkq, blkk, is_causal, pv_mode, dtype,
-                   cu_seqlens_q, cu_seqlens_k, plan, total_q, w.qs_sh, w.ks_sh, w.panel_sh, m, lse_off, qr, stream);
+                   Skv, D, fuse_q ? q_sb : qi_sb, fuse_q ? q_sh : qi_sh, fuse_q ? q_sn : qi_sn, ki_sb, ki_sh, ki_sn, o_sb, o_sh,
+                   o_sn, blkq, blkk, is_causal, pv_mode, dtype, cu_seqlens_q, cu_seqlens_k, plan, total_q, w.qs_sh, w.ks_sh,
+                   w.panel_sh, m, lse_off, qr, stream);
 }
 
 }  // extern "C"

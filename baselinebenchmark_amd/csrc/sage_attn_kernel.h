@@ -758,7 +758,8 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
   if constexpr (MSUM) lsum = osum[0];
   else lsum = xchg32_sum(lsum);
   const float den = RSUM ? osum[0] : lsum;
-  const float inv = den > 0.f ? 1.0f / den : 0.f;
+  const bool live = den > 0.f;   // a row with no visible key (or no keys at all) yields zeros
+  const float inv = live ? 1.0f / den : 0.f;
   if (my_row < Lq) {
     if (a.lse && h == 0) {
       // lse_offset: what K smoothing removed from every logit of this row (q . k_mean, base-2 units)
@@ -794,7 +795,8 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
 #pragma unroll
           for (int i = 0; i < 4; i++) {
             f[i] = o[dt][4 * q4 + i] * inv;
-            if constexpr (PV == 1) f[i] *= vs_lds[d + i];
+            // (the V scales are not read for a dead row: with no keys at all nothing ever wrote them)
+            if constexpr (PV == 1) f[i] = live ? f[i] * vs_lds[d + i] : 0.f;
           }
           u16 hv[4];
 #pragma unroll

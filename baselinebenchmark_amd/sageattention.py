@@ -330,7 +330,8 @@ def _apply_recipe(quant_recipe, BLKQ, BLKK, pv_mode):
 
 @torch.no_grad()
 def sageattn(q, k, v, tensor_layout="HND", is_causal=False, sm_scale=None, smooth_k=True, pv_mode=None,
-             BLKQ=128, BLKK=64, return_lse=False, qk_quant_dtype="int8", quant_recipe=None, attn_mask=None, **kwargs):
+             BLKQ=128, BLKK=64, return_lse=False, qk_quant_dtype="int8", quant_recipe=None, attn_mask=None,
+             cu_seqlens_q=None, cu_seqlens_k=None, max_seqlen_q=None, max_seqlen_k=None, **kwargs):
     """Quantise + attend in one call: out = softmax(q k^T * sm_scale [causal | + attn_mask]) v.
 
     Returns ``out`` (q's shape and dtype), or ``(out, lse)`` with ``return_lse=True`` where lse is
@@ -341,12 +342,32 @@ def sageattn(q, k, v, tensor_layout="HND", is_causal=False, sm_scale=None, smoot
     ``quant_recipe`` (the keyword of sage_attention_benchmark_compare.py:300-313): (Q rows, K rows, -1, 1) sets the
     scale blocks and selects per-channel FP8 V, e.g. the external recipe (128, 16, -1, 1); without it ``BLKQ`` /
     ``BLKK`` / ``pv_mode`` ("fp16" by default) apply.
+    ``cu_seqlens_q`` / ``cu_seqlens_k`` (int32 [nseq+1] on the device) switch to packed variable-length batches:
+    q is then [total_q, Hq, D], k and v [total_k, Hkv, D], ``tensor_layout`` is not consulted, ``max_seqlen_q`` /
+    ``max_seqlen_k`` bound the sequence lengths (derived from cu_seqlens, with one host synchronisation, when left
+    out), and lse comes back as [Hq, total_q]; see sageattn_varlen, which this call is then identical to.
     """
     if qk_quant_dtype != "int8":
         raise NotImplementedError("only INT8 Q/K quantisation is implemented")
     if kwargs:
         raise TypeError(f"unexpected arguments: {sorted(kwargs)}")
     BLKQ, BLKK, pv_mode = _apply_recipe(quant_recipe, BLKQ, BLKK, pv_mode)
+    if cu_seqlens_q is not None or cu_seqlens_k is not None:
+        if attn_mask is not None:
+            raise NotImplementedError("attn_mask is not supported for packed batches")
+        cu_seqlens_k = cu_seqlens_q if cu_seqlens_k is None else cu_seqlens_k
+        cu_seqlens_q = cu_seqlens_k if cu_seqlens_q is None else cu_seqlens_q
+        _check_cu("cu_seqlens_q", cu_seqlens_q, q.device)
+        _check_cu("cu_seqlens_k", cu_seqlens_k, q.device)
+        if max_seqlen_q is None:
+            max_seqlen_q = int((cu_seqlens_q[1:] - cu_seqlens_q[:-1]).max().item())
+        if max_seqlen_k is None:
+            max_seqlen_k = int((cu_seqlens_k[1:] - cu_seqlens_k[:-1]).max().item())
+        return sageattn_varlen(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, is_causal=is_causal,
+                               sm_scale=sm_scale, smooth_k=smooth_k, pv_mode=pv_mode, BLKQ=BLKQ, BLKK=BLKK,
+                               return_lse=return_lse)
+    if max_seqlen_q is not None or max_seqlen_k is not None:
+        raise ValueError("max_seqlen_q / max_seqlen_k only apply together with cu_seqlens_q / cu_seqlens_k")
     for name, t in (("q", q), ("k", k), ("v", v)):
         _check_float(name, t)
     if not (q.dtype == k.dtype == v.dtype) or not (q.device == k.device == v.device):

@@ -210,6 +210,8 @@ int sage_attn_fwd_masked(const int8_t* q, const int8_t* k, const void* v_panels,
  * (cu_seqlens_* != NULL; total_q/total_k = packed row counts).
  * lse (may be NULL) receives the base-2 log-sum-exp of the logits of the ORIGINAL k: with smooth_k the
  * term q . k_mean that smoothing removed from every logit of a row is added back.
+ * q, k, v and out may be arbitrary strided views (16-byte aligned rows, contiguous head_dim), e.g. slices of a
+ * fused QKV buffer: the INT8 copies inside the workspace use dense strides of their own.
  */
 size_t sage_sageattn_workspace_bytes(int B, int Hq, int Hkv, int Sq, int Skv, int D,
                                      int blkq, int blkk, int pv_mode, int total_q, int total_k,
@@ -247,21 +249,6 @@ int sage_sageattn_masked(const void* q, const void* k, const void* v, void* out,
                          const void* attn_mask, int mask_kind,
                          int64_t m_sb, int64_t m_sh, int64_t m_sm, int64_t m_sn,
                          sage_stream_t stream);
-
-/*
- * Hardware-rate micro-benchmarks (no counterpart in the reference: a measurement aid for the roofline
- * denominators).  kind: 0 v_mfma_i32_32x32x32_i8 from registers, 1 v_mfma_f32_32x32x64_f8f6f4 (fp8) from
- * registers, 2 LDS reads (ds_read_b128), 3 / 4 the two MFMAs with every operand fragment read from LDS
- * as the attention kernel does, 5 v_fma_f32, 6 v_exp_f32, 7 v_cvt_pk_fp8_f32, 8 the softmax mix (per
- * score one fma, one exp2, half a packed fp8 conversion).  sage_microbench launches `grid` workgroups
- * (one per compute unit is the intended use) of 4 * waves_per_simd wavefronts (1, 2 or 4 per SIMD),
- * `iters` iterations each; the caller times the launch.  sage_microbench_units gives the work of one
- * wavefront per iteration: operations (a multiply-add counts 2), bytes, or instructions.
- * `sink` takes grid * 1024 ints.
- */
-double sage_microbench_units(int kind);
-int sage_microbench(int kind, int grid, int waves_per_simd, int iters, void* sink, size_t sink_bytes,
-                    sage_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -11,8 +11,9 @@ Pinning status of each oracle function (what independent evidence fixes it):
   guard of backends/_hygon/ops/sageattention/sageattention_triton.py:35.  The
   reference holds no golden vectors for it; pinned by closed-form invariants
   (arg-max element -> +-127, |x - q*scale| <= scale/2, round-half-away ties, masked
-  tail rows) and a second, independent big-rational restatement on small tiles
-  (tests/test_oracle_quant.py) plus the C restatement ``oracle/sage_oracle.c``.
+  tail rows), a second, independent big-rational restatement on small tiles
+  (tests/test_oracle_quant.py) and golden vectors that the reference's own quantiser
+  produced (tests/golden/quant_golden.npz, written by tests/golden/make_quant_golden.py).
 * ``quant.k_mean`` -- the reference never computes the K mean (it is only an argument,
   quant_per_block.py:53-54): **parity unpinned**; definition stated in its docstring.
 * ``quant.quant_v_fp8`` -- FP8 P.V is not in the reference's own kernels: **parity
@@ -25,4 +26,8 @@ Pinning status of each oracle function (what independent evidence fixes it):
   torch.nn.functional.scaled_dot_product_attention and brute-force loops on tiny
   shapes.  Its causal / varlen extensions are not in the reference: **parity unpinned**
   there, pinned by SDPA ``is_causal=True`` and a per-sequence loop.
+* ``fp8_model.fp8_attention_model`` -- the arithmetic of this build's FP8 P.V kernel (e4m3 P
+  and V, lazily moved reference maximum, denominator from the rounded probabilities); the
+  reference has no FP8 kernel: **parity unpinned** there, pinned by scalar-loop closed forms,
+  exact invariants and closeness to ``sage_reference`` (tests/test_oracle_fp8_model.py).
 """

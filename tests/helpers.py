@@ -26,3 +26,32 @@ def golden_case(g, name):
     for key in ("qi", "qs", "ki", "ks"):
         d[key] = torch.from_numpy(g[f"{name}.{key}"].copy())
     return d
+
+
+def sageattn_cabi(q, k, v, out, *, layout="HND", is_causal=False, pv="fp16", BLKQ=128, BLKK=64, smooth_k=True, sm_scale=None,
+                  lse=None, workspace=None):
+    """sage_sageattn straight through ctypes, with the tensors' own strides (any view whose last
+    axis is contiguous), bypassing the Python shim's contiguity checks.  Returns the C return code."""
+    import ctypes
+    from baselinebenchmark_amd import _cabi
+
+    lib = _cabi.lib()
+
+    def lay(t):
+        if layout == "HND":
+            return t.shape[0], t.shape[1], t.shape[2], t.shape[3], t.stride(0), t.stride(1), t.stride(2)
+        return t.shape[0], t.shape[2], t.shape[1], t.shape[3], t.stride(0), t.stride(2), t.stride(1)
+
+    B, Hq, Sq, D, qsb, qsh, qsn = lay(q)
+    _, Hkv, Skv, _, ksb, ksh, ksn = lay(k)
+    _, _, _, _, vsb, vsh, vsn = lay(v)
+    _, _, _, _, osb, osh, osn = lay(out)
+    pvm = _cabi.PV_FP8 if pv == "fp8" else _cabi.PV_FP16
+    dt = _cabi.DT_BF16 if q.dtype == torch.bfloat16 else _cabi.DT_F16
+    P = lambda t: ctypes.c_void_p(0 if t is None else t.data_ptr())
+    stream = ctypes.c_void_p(torch.cuda.current_stream(q.device).cuda_stream)
+    tail = (B, Hq, Hkv, Sq, Skv, D, qsb, qsh, qsn, ksb, ksh, ksn, vsb, vsh, vsn, osb, osh, osn, dt, BLKQ, BLKK,
+            float(D ** -0.5 if sm_scale is None else sm_scale), int(is_causal), int(smooth_k), pvm, None, None, 0, 0, stream)
+    nbytes = lib.sage_sageattn_workspace_bytes(B, Hq, Hkv, Sq, Skv, D, BLKQ, BLKK, pvm, 0, 0, 0)
+    ws = workspace if workspace is not None else torch.empty(max(nbytes, 256), device=q.device, dtype=torch.uint8)
+    return lib.sage_sageattn(P(q), P(k), P(v), P(out), P(lse), P(ws), ws.numel(), *tail)

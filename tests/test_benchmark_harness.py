@@ -71,6 +71,8 @@ def test_hw_rate_microbenchmarks_run_and_are_plausible():
     """The micro-benchmarks behind the measured roofline denominators: every kind runs through the C ABI and the two
     MFMA instructions reach at least half of the datasheet rate from registers (they measure 80-95 % on the box)."""
     from baselinebenchmark_amd.benchmarks import hw_rates
+    if not hw_rates.LIB_PATH.exists():
+        pytest.skip("tool library absent (python -m baselinebenchmark_amd.build --tools)")
     rows = hw_rates.run(iters_mfma=500, iters_valu=2000)
     assert len(rows) == 3 * len(hw_rates.KINDS)
     best = {}
@@ -91,7 +93,7 @@ def test_tile_timing_tool_reports_the_intervals_of_a_workgroup():
     from baselinebenchmark_amd.build import TIMING_LIB
     ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     if not TIMING_LIB.exists():
-        pytest.skip("timing build absent (python -m baselinebenchmark_amd.build --timing)")
+        pytest.skip("timing build absent (python -m baselinebenchmark_amd.build --tools)")
     code = ("from baselinebenchmark_amd.benchmarks import tile_timing as t\n"
             "rows, tiles = t.measure(2, 4, 4096, 128, True, launches=2)\n"
             "import json; print(json.dumps({'rows': rows, 'tiles': tiles}))\n")

@@ -392,3 +392,31 @@ def test_sageattn_with_the_external_quant_recipe():
     assert torch.equal(out, same)
     m = oa.metrics(out.cpu().float(), oa.sdpa_fp32(q, k, v, "HND", False))
     assert m["finite"] and m["cosine"] >= 0.999, m
+
+
+def test_config1_full_size_against_the_reference_formula():
+    """BASELINE config 1 at its full size (B4 H32 S4096 D128 bf16, causal, Q blk 128 / K blk 64, FP16 P.V, K with a
+    per-channel offset ~ N(0,4) that K smoothing has to remove) through the one-call entry point.  One head is only
+    4096 x 4096 logits, so three (batch, head) slices are checked in full against the reference formula on operands
+    quantised by the oracle (relative RMSE < 4e-3: bf16 output rounding is 1.1e-3 rms) and against FP32 SDPA on the
+    raw inputs (cosine >= 0.999); plus determinism and head independence, bit for bit."""
+    from baselinebenchmark_amd import workloads
+    from oracle import quant as oq
+    w = workloads.make("c1", device=DEV)
+    assert w.kwargs["pv_mode"] == "fp16" and w.kwargs["is_causal"] and (w.kwargs["BLKQ"], w.kwargs["BLKK"]) == (128, 64)
+    out = sa.sageattn(w.q, w.k, w.v, **w.kwargs)
+    assert tuple(out.shape) == (4, 32, 4096, 128) and torch.isfinite(out.float()).all()
+    assert torch.equal(out, sa.sageattn(w.q, w.k, w.v, **w.kwargs))
+    perm = torch.randperm(32, generator=torch.Generator().manual_seed(7)).to(DEV)
+    assert torch.equal(sa.sageattn(w.q[:, perm].contiguous(), w.k[:, perm].contiguous(), w.v[:, perm].contiguous(), **w.kwargs),
+                       out[:, perm])
+    for b, h in ((0, 0), (2, 17), (3, 31)):
+        q1, k1, v1 = (t[b:b + 1, h:h + 1].cpu() for t in (w.q, w.k, w.v))
+        assert k1.float().mean(dim=2).abs().max().item() > 1.0          # the offset is there
+        qi, qs, ki, ks = oq.per_block_int8(q1, k1, km=oq.k_mean(k1), BLKQ=128, BLKK=64)
+        ref, _ = oa.sage_reference(qi, ki, v1, qs, ks, "HND", 128, 64, is_causal=True)
+        got = out[b:b + 1, h:h + 1].cpu().float()
+        m = oa.metrics(got, ref)
+        assert m["rel_rmse"] < 4e-3 and m["cosine"] >= 0.9999, (b, h, m)
+        ms = oa.metrics(got, oa.sdpa_fp32(q1, k1, v1, "HND", True))
+        assert ms["cosine"] >= 0.999, (b, h, ms)

@@ -81,3 +81,54 @@ def test_many_heads_few_rows_exercises_the_head_to_xcd_mapping():
         out, _ = sa.forward(qi, ki, v.to(DEV), qs, ks)
         ref, _ = oa.sage_reference(qi.cpu(), ki.cpu(), v, qs.cpu(), ks.cpu(), "HND", 128, 64)
         assert oa.metrics(out.cpu().float(), ref)["rel_rmse"] < 2e-3
+
+
+@pytest.mark.parametrize("pv", ["fp16", "fp8"])
+def test_no_keys_at_all_gives_zeros_and_minus_infinity(pv):
+    """Skv == 0 with Sq > 0: every row is a row with no visible key (out = 0, LSE = -inf), and nothing of K, V or their
+    scales may be read -- the FP8 V scales in particular are never written in that case."""
+    q = torch.randn((2, 4, 77, 128), dtype=torch.float16, device=DEV)
+    kv = torch.empty((2, 2, 0, 128), dtype=torch.float16, device=DEV)
+    junk = torch.full((1 << 20,), float("nan"), device=DEV)   # poison what the allocator hands out next
+    del junk
+    out, lse = sa.sageattn(q, kv, kv, pv_mode=pv, return_lse=True)
+    assert tuple(out.shape) == tuple(q.shape) and torch.count_nonzero(out).item() == 0
+    assert torch.isinf(lse).all() and (lse < 0).all()
+    out = sa.sageattn(q, kv, kv, pv_mode=pv)
+    assert torch.count_nonzero(out).item() == 0
+    qi, qs, ki, ks = sa.per_block_int8(q, kv)
+    o2, l2 = sa.forward(qi, ki, kv, qs, ks, return_lse=True, pv_mode=pv)
+    assert torch.count_nonzero(o2).item() == 0 and torch.isinf(l2).all()
+
+
+@pytest.mark.parametrize("pv,causal,lse", [("fp8", True, False), ("fp16", False, True)])
+def test_strided_views_of_a_fused_qkv_buffer_through_the_c_abi(pv, causal, lse):
+    """q, k and v as slices of one [B, S, 3, H, D] buffer (row stride 3*H*D) and a strided output: the INT8 copies the
+    one-call pipeline makes inside its workspace must not inherit those strides.  The workspace is exactly the size
+    the library asks for and sits in the middle of a guarded allocation, so a stray write is seen."""
+    from baselinebenchmark_amd import _cabi
+    from tests.helpers import sageattn_cabi
+    B, S, H, D = 2, 300, 4, 128
+    g = torch.Generator().manual_seed(31)
+    qkv = torch.randn((B, S, 3, H, D), generator=g).to(torch.bfloat16).to(DEV)
+    q, k, v = qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2]          # NHD views, row stride 3*H*D
+    assert not q.is_contiguous()
+    obuf = torch.zeros((B, S, 2, H, D), dtype=torch.bfloat16, device=DEV)
+    out = obuf[:, :, 1]
+    need = _cabi.lib().sage_sageattn_workspace_bytes(B, H, H, S, S, D, 64, 128, _cabi.PV_FP8 if pv == "fp8" else _cabi.PV_FP16, 0, 0, 0)
+    guard = 1 << 16
+    buf = torch.full((need + 2 * guard + 256,), 0x5A, dtype=torch.uint8, device=DEV)
+    base = (-(buf.data_ptr() + guard)) % 256 + guard
+    ws = buf[base:base + need]
+    lse_t = torch.empty((B, H, S), dtype=torch.float32, device=DEV) if lse else None
+    rc = sageattn_cabi(q, k, v, out, layout="NHD", is_causal=causal, pv=pv, BLKQ=64, BLKK=128, workspace=ws, lse=lse_t)
+    assert rc == 0, _cabi.lib().sage_last_error().decode()
+    torch.cuda.synchronize()
+    assert (buf[:base] == 0x5A).all() and (buf[base + need:] == 0x5A).all()
+    assert torch.count_nonzero(obuf[:, :, 0]).item() == 0
+    ref = sa.sageattn(q.contiguous(), k.contiguous(), v.contiguous(), tensor_layout="NHD", is_causal=causal, pv_mode=pv,
+                      BLKQ=64, BLKK=128, return_lse=lse)
+    if lse:
+        ref, ref_lse = ref
+        assert torch.allclose(lse_t * 0.6931471805599453, ref_lse, rtol=0, atol=1e-6)
+    assert torch.equal(out.contiguous().view(torch.int16), ref.view(torch.int16))

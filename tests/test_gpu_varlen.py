@@ -131,3 +131,23 @@ def test_varlen_lse_is_the_per_sequence_logsumexp(smooth, causal):
             logits = logits.masked_fill(~torch.ones(L, L, dtype=torch.bool).tril(), -float("inf"))
         ref = torch.logsumexp(logits, dim=-1)
         assert (lse[:, a:b].cpu().double() - ref).abs().max().item() < 6e-2, (i, L)     # INT8 noise on the logits
+
+
+def test_sageattn_with_cu_seqlens_is_the_packed_call():
+    """The entry point as the harness spells it -- sageattn(q, k, v, ..., cu_seqlens_q=, cu_seqlens_k=, max_seqlen_q=,
+    max_seqlen_k=) (call shape of backends/_metax/benchmarks/sage_attention/benchmark.py:29 plus the optional packed
+    arguments) -- is bit-identical to sageattn_varlen, with and without LSE and with the lengths left out."""
+    lens = [300, 1, 129, 1025]
+    q, k, v, cu = _packed(lens, 8, 2, 128, torch.bfloat16, 11)
+    qd, kd, vd, cud = q.to(DEV), k.to(DEV), v.to(DEV), cu.to(DEV)
+    kw = dict(is_causal=True, pv_mode="fp8", BLKQ=64, BLKK=128)
+    ref, ref_lse = sa.sageattn_varlen(qd, kd, vd, cud, cud, max(lens), max(lens), return_lse=True, **kw)
+    out, lse = sa.sageattn(qd, kd, vd, cu_seqlens_q=cud, cu_seqlens_k=cud, max_seqlen_q=max(lens), max_seqlen_k=max(lens),
+                           return_lse=True, **kw)
+    assert torch.equal(out, ref) and torch.equal(lse, ref_lse)
+    out2 = sa.sageattn(qd, kd, vd, cu_seqlens_q=cud, cu_seqlens_k=cud, **kw)          # lengths derived from cu_seqlens
+    assert torch.equal(out2, sa.sageattn_varlen(qd, kd, vd, cud, cud, max(lens), max(lens), **kw))
+    with pytest.raises(NotImplementedError):
+        sa.sageattn(qd, kd, vd, cu_seqlens_q=cud, attn_mask=torch.ones((1, 1), dtype=torch.bool, device=DEV))
+    with pytest.raises(ValueError):
+        sa.sageattn(qd.unsqueeze(0), kd.unsqueeze(0), vd.unsqueeze(0), tensor_layout="NHD", max_seqlen_q=5)
