@@ -47,6 +47,10 @@ SIGNATURES = {
     "sage_sageattn": (c_int, [_P, _P, _P, _P, _P, _P, c_size_t, _I, _I, _I, _I, _I, _I,
                               _L, _L, _L, _L, _L, _L, _L, _L, _L, _L, _L, _L,
                               _I, _I, _I, c_double, _I, _I, _I, _P, _P, _I, _I, _P]),
+    "sage_sageattn_static_capacity": (c_size_t, []),
+    "sage_sageattn_static": (c_int, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I,
+                                     _L, _L, _L, _L, _L, _L, _L, _L, _L, _L, _L, _L,
+                                     _I, _I, _I, c_double, _I, _I, _I, _P, _P, _I, _I, _P]),
     "sage_sageattn_masked": (c_int, [_P, _P, _P, _P, _P, _P, c_size_t, _I, _I, _I, _I, _I, _I,
                                      _L, _L, _L, _L, _L, _L, _L, _L, _L, _L, _L, _L,
                                      _I, _I, _I, c_double, _I, _I, _I, _P, _P, _I, _I,

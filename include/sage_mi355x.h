@@ -250,6 +250,33 @@ int sage_sageattn_masked(const void* q, const void* k, const void* v, void* out,
                          int64_t m_sb, int64_t m_sh, int64_t m_sm, int64_t m_sn,
                          sage_stream_t stream);
 
+/*
+ * sage_sageattn for callers that cannot allocate device memory or carry a workspace (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid allocation).  It has no counterpart in the reference.
+ * Same arguments and results as sage_sageattn minus `workspace`/`workspace_bytes`: the intermediates (INT8 K,
+ * scales, K mean, V panels, statistics partials, the packed-batch plan, INT8 Q where a separate pass is needed)
+ * live in an array of SAGE_STATIC_SCRATCH_BYTES that is part of the library's device image, one copy per GPU,
+ * held until the process ends.  The call allocates and frees nothing and does not synchronise.
+ * Limit: sage_sageattn_workspace_bytes(...) of the problem must not exceed sage_sageattn_static_capacity()
+ * (= SAGE_STATIC_SCRATCH_BYTES); larger problems return SAGE_EWORKSPACE and launch nothing.
+ * All calls on one GPU share that GPU's array: calls that may overlap on one GPU (different streams, or host
+ * threads without ordering between their streams) race; serialise them or use sage_sageattn.  The array keeps
+ * the previous call's contents; every intermediate is rewritten before it is read, so nothing needs clearing.
+ */
+#define SAGE_STATIC_SCRATCH_BYTES (64u << 20)
+size_t sage_sageattn_static_capacity(void);
+int sage_sageattn_static(const void* q, const void* k, const void* v, void* out, float* lse,
+                         int B, int Hq, int Hkv, int Sq, int Skv, int D,
+                         int64_t q_sb, int64_t q_sh, int64_t q_sn,
+                         int64_t k_sb, int64_t k_sh, int64_t k_sn,
+                         int64_t v_sb, int64_t v_sh, int64_t v_sn,
+                         int64_t o_sb, int64_t o_sh, int64_t o_sn,
+                         int dtype, int blkq, int blkk, double sm_scale, int is_causal, int smooth_k,
+                         int pv_mode,
+                         const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+                         int total_q, int total_k,
+                         sage_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

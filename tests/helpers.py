@@ -29,8 +29,8 @@ def golden_case(g, name):
 
 
 def sageattn_cabi(q, k, v, out, *, layout="HND", is_causal=False, pv="fp16", BLKQ=128, BLKK=64, smooth_k=True, sm_scale=None,
-                  lse=None, workspace=None):
-    """sage_sageattn straight through ctypes, with the tensors' own strides (any view whose last
+                  static=False, lse=None, workspace=None):
+    """sage_sageattn / sage_sageattn_static straight through ctypes, with the tensors' own strides (any view whose last
     axis is contiguous), bypassing the Python shim's contiguity checks.  Returns the C return code."""
     import ctypes
     from baselinebenchmark_amd import _cabi
@@ -52,6 +52,8 @@ def sageattn_cabi(q, k, v, out, *, layout="HND", is_causal=False, pv="fp16", BLK
     stream = ctypes.c_void_p(torch.cuda.current_stream(q.device).cuda_stream)
     tail = (B, Hq, Hkv, Sq, Skv, D, qsb, qsh, qsn, ksb, ksh, ksn, vsb, vsh, vsn, osb, osh, osn, dt, BLKQ, BLKK,
             float(D ** -0.5 if sm_scale is None else sm_scale), int(is_causal), int(smooth_k), pvm, None, None, 0, 0, stream)
+    if static:
+        return lib.sage_sageattn_static(P(q), P(k), P(v), P(out), P(lse), *tail)
     nbytes = lib.sage_sageattn_workspace_bytes(B, Hq, Hkv, Sq, Skv, D, BLKQ, BLKK, pvm, 0, 0, 0)
     ws = workspace if workspace is not None else torch.empty(max(nbytes, 256), device=q.device, dtype=torch.uint8)
     return lib.sage_sageattn(P(q), P(k), P(v), P(out), P(lse), P(ws), ws.numel(), *tail)
