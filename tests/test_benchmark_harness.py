@@ -105,3 +105,20 @@ def test_tile_timing_tool_reports_the_intervals_of_a_workgroup():
     for name, vals in doc["rows"].items():
         assert len(vals) == 7 and all(v > 0 for v in vals), (name, vals)
         assert vals[4] > 0.5 * sum(vals), (name, vals)
+
+
+@pytest.mark.gpu
+def test_cpp_driver_calls_the_c_abi_directly():
+    """sage_bench: a C++ program (no Python, no torch) that links libsage_mi355x.so, runs sage_sageattn and
+    sage_sageattn_static on one stream with its own device buffers, gates the result and prints the table row."""
+    import subprocess
+    from baselinebenchmark_amd.build import CABI_BENCH
+    if not CABI_BENCH.exists():
+        pytest.skip("C++ driver absent (python -m baselinebenchmark_amd.build --tools)")
+    for extra in ([], ["--static", "1"], ["--layout", "NHD", "--pv", "fp16", "--dtype", "fp16", "--kv-heads", "2"]):
+        res = subprocess.run([str(CABI_BENCH), "--batch", "1", "--heads", "4", "--kv-heads", "4", "--seq", "1024", "--warmup", "2",
+                              "--rep", "3", *extra], capture_output=True, text=True, timeout=120)
+        assert res.returncode == 0, (extra, res.stdout, res.stderr)
+        head, row = res.stdout.strip().splitlines()[-2:]
+        cols = dict(zip(head.split("\t"), row.split("\t")))
+        assert cols["gate"] == "PASS" and float(cols["latency_ms"]) > 0 and cols["backend"] == "mi355x_hip_int8_qk_fp8_fp16_pv"
