@@ -29,7 +29,7 @@ def _read():
     if fn is None:
         raise SystemExit(f"{LIB_PATH} is not a timing build: run `python -m baselinebenchmark_amd.build --timing` and set "
                          "SAGE_MI355X_LIB to csrc/libsage_mi355x_timing.so")
-    buf = (ctypes.c_ulonglong * 32)()
+    buf = (ctypes.c_ulonglong * 48)()
     if fn(buf) != 0:
         raise RuntimeError("sage_tile_timing failed")
     return list(buf)
@@ -51,6 +51,11 @@ def measure(B, H, S, D, causal, dtype=torch.bfloat16, pv_mode="fp8", blkq=64, bl
         n = max(d[cls * 8 + 7], 1)
         rows[name] = [d[cls * 8 + i] * TICK_NS / n for i in range(7)]
     tiles = d[24] / max(d[7], 1)
+    # main loop of the FP8 kernels, per period and group: first phase, wait at the odd barrier, second phase, wait at the
+    # even barrier (group 0: matrix phase first; group 1: vector phase first)
+    for g in (0, 1):
+        n = max(d[40 + g], 1)
+        rows[f"group {g} phases"] = [d[32 + 4 * g + k] * TICK_NS / n for k in range(4)]
     return rows, tiles
 
 
@@ -65,6 +70,10 @@ def main():
         rows, tiles = measure(B, H, S, D, bool(int(causal)))
         print(f"B{B} H{H} S{S} D{D} causal={bool(int(causal))}: {tiles:.1f} K tiles per workgroup", flush=True)
         for name, vals in rows.items():
+            if len(vals) == 4:
+                print(f"  {name:17s} per period {sum(vals):6.0f} ns | first phase {vals[0]:.0f}, odd barrier {vals[1]:.0f}, "
+                      f"second phase {vals[2]:.0f}, even barrier {vals[3]:.0f}", flush=True)
+                continue
             parts = ", ".join(f"{lbl} {v:.0f}" for lbl, v in zip(INTERVALS, vals))
             print(f"  {name:17s} total {sum(vals):8.0f} ns | {parts} | main loop per tile {vals[4] / max(tiles, 1e-9):.0f}", flush=True)
 

@@ -31,8 +31,18 @@
 //     are in different groups, so each SIMD always has matrix work and vector work to overlap.
 #pragma once
 #include "sage_launch.h"
+#include <atomic>
 #include <cstdlib>
 // Bit of the wavefront index that picks the group: wavefronts w and w + 4 share a SIMD.
+#ifndef SAGE_KPF
+#define SAGE_KPF 4
+#endif
+#ifndef SAGE_VPF
+#define SAGE_VPF 3
+#endif
+#ifndef SAGE_REQ_GROUP
+#define SAGE_REQ_GROUP 0
+#endif
 #ifndef SAGE_GSH
 #define SAGE_GSH 2
 #endif
@@ -117,10 +127,15 @@ constexpr int attn_lds_bytes() { return attn_tile_lds_bytes<D, NW, BN, PV, CAUSA
 // tile on the constant-rate 100 MHz counter and adds the seven intervals to per-class sums (class 0 =
 // first wavefront, 1 = last, 2 = the others): [class][0..6] intervals in ticks, [class][7] wavefronts,
 // [3][0] = tiles.  SAGE_T(k, x) pins stamp k after the computation of x.
+// Also, in the main loop of the FP8 kernels, four stamps per period (after the even barrier, before and after the odd
+// barrier, at the end of the period) are summed per group: [32 + 4 g + k] = ticks from stamp k to the next one (k = 0:
+// first phase of the period, 1: wait at the odd barrier, 2: second phase, 3: wait at the even barrier), [40 + g] = periods.
 #ifdef SAGE_TIMING
-static __device__ unsigned long long g_tile_timing[32];
+static __device__ unsigned long long g_tile_timing[48];
+#define SAGE_PH(k) do { const long long t_ = __builtin_amdgcn_s_memrealtime(); if (ph_last) ph_sum[((k) + 3) & 3] += t_ - ph_last; ph_last = t_; if ((k) == 0) ph_n++; } while (0)
 #define SAGE_T(k, x) do { asm volatile("" : "+v"(x)); sage_ts[k] = __builtin_amdgcn_s_memrealtime(); } while (0)
 #else
+#define SAGE_PH(k) do { } while (0)
 #define SAGE_T(k, x) do { } while (0)
 #endif
 // MASK: 0 none, 1 boolean keep-mask (bytes), 2 additive fp32 bias in base-2 score units
@@ -157,6 +172,8 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
 #ifdef SAGE_TIMING
   long long sage_ts[8];
   for (int i = 0; i < 8; i++) sage_ts[i] = __builtin_amdgcn_s_memrealtime();
+  long long ph_last = 0, ph_sum[4] = {0, 0, 0, 0};
+  int ph_n = 0;
 #endif
   const int tid = threadIdx.x, lane = tid & 63;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);  // wavefront index: uniform, keep it scalar
@@ -275,9 +292,13 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
   float* vs_lds = reinterpret_cast<float*>(smem + attn_tile_lds_bytes<D, NW, BN, PV, CAUSAL, QF>());
   if constexpr (PV == 1) {
     if (w < D / 64) {
-      const __amdgpu_buffer_rsrc_t vsrsrc =
-          __builtin_amdgcn_make_buffer_rsrc((void*)(a.vs + ((int64_t)b * a.Hkv + kvh) * D), 0, D * 4, 0x00020000);
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(vsrsrc, (__attribute__((address_space(3))) void*)(vs_lds + 64 * w), 4, lane * 4, w * 256, 0, 0);
+      if (Lk > 0) {
+        const __amdgpu_buffer_rsrc_t vsrsrc =
+            __builtin_amdgcn_make_buffer_rsrc((void*)(a.vs + ((int64_t)b * a.Hkv + kvh) * D), 0, D * 4, 0x00020000);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(vsrsrc, (__attribute__((address_space(3))) void*)(vs_lds + 64 * w), 4, lane * 4, w * 256, 0, 0);
+      } else {
+        vs_lds[64 * w + lane] = 1.0f;   // no keys: nothing ever wrote the scales, and 0 * garbage must stay 0
+      }
     }
   }
 
@@ -345,24 +366,31 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
     const float rcp = 1.0f / scale;
     const uint32_t sbits = __builtin_bit_cast(uint32_t, scale);
     const bool fast = ((sbits & 0x7fffffu) != 0x7fffffu) && scale < 1.0e30f;
+    // (one uniform branch around the whole tile, not one per element: the two quotients are the same numbers)
+    auto quantise_rows = [&](auto quotient) __attribute__((always_inline)) {
 #pragma unroll
-    for (int ks = 0; ks < KS; ks++) {
-      uint32_t packed[4] = {0, 0, 0, 0};
+      for (int ks = 0; ks < KS; ks++) {
+        uint32_t packed[4] = {0, 0, 0, 0};
 #pragma unroll
-      for (int i = 0; i < 16; i++) {
-        float z = fast ? div_by_uniform(x[ks][i], scale, rcp) : x[ks][i] / scale;
-        z = z + __builtin_copysignf(0.5f, z);
-        int qv = (int)z;
-        packed[i >> 2] |= (uint32_t)(qv & 0xff) << (8 * (i & 3));
+        for (int i = 0; i < 16; i++) {
+          float z = quotient(x[ks][i]);
+          z = z + __builtin_copysignf(0.5f, z);
+          int qv = (int)z;
+          packed[i >> 2] |= (uint32_t)(qv & 0xff) << (8 * (i & 3));
+        }
+        qreg[ks] = v4i{(int)packed[0], (int)packed[1], (int)packed[2], (int)packed[3]};
       }
-      qreg[ks] = v4i{(int)packed[0], (int)packed[1], (int)packed[2], (int)packed[3]};
-    }
+    };
+    if (fast) quantise_rows([&](float v) { return div_by_uniform(v, scale, rcp); });
+    else quantise_rows([&](float v) { return v / scale; });
     qscale = scale;
   }
 
 
-  // With two periods of lead the second K tile follows as soon as the raw Q rows are out of the way.
-  if (LEAD == 2 && ntiles > 1) load_k(1, dw_self);
+  // The other K tiles of the lead follow as soon as the raw Q rows are out of the way.
+#pragma unroll
+  for (int t = 1; t < LEAD; t++)
+    if (t < ntiles) load_k(t, dw_self);
 
   v16i bias;
 #pragma unroll
@@ -404,7 +432,7 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
     // K fragments run KPF MFMAs ahead of their use so that no MFMA waits for the LDS read issued
     // just before it; the k-step is the outer index so that consecutive MFMAs hit different accumulators.
     {
-      constexpr int NF = NT * KS, KPF = 4;
+      constexpr int NF = NT * KS, KPF = SAGE_KPF;
       auto kfrag = [&](int i) {
         const int nt = i % NT, ks = i / NT, n = 32 * nt + m;
         return *reinterpret_cast<const v4i*>(kbuf + n * D + 16 * ((2 * ks + h) ^ kswz<D>(n)));
@@ -596,7 +624,7 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
   auto pv = [&](int j) {
     const uint8_t* vbuf = vslot(j);
     if constexpr (PV == 1) {
-      constexpr int NV = (BN / 64) * DTN, VPF = 3;
+      constexpr int NV = (BN / 64) * DTN, VPF = SAGE_VPF;
       auto vfrag = [&](int i) {
         const uint8_t* vp0 = vbuf + ((i * 2) * 64 + lane) * 16;
         v4i lo = *reinterpret_cast<const v4i*>(vp0);
@@ -695,8 +723,9 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
     // V(j+LEAD-1), LEAD periods before their first use (a tile that has to come from HBM takes longer than one
     // period), into the slots whose last readers finished a barrier ago; with LEAD = 2, V(0) goes first in
     // period 0 and the requests of the last period may still be in flight at a barrier.
-    auto request_tiles = [&](int j) {
-      if (LEAD == 2 && j == 0) { load_v(0, 0); load_v(0, PARTNER); }
+    auto first_value_tile = [&]() { load_v(0, 0); load_v(0, PARTNER); };
+    auto request_tiles = [&](int j, bool with_first_value = true) {
+      if (LEAD == 2 && j == 0 && with_first_value) first_value_tile();
       if (j + LEAD < ntiles) { load_k(j + LEAD, 0); load_k(j + LEAD, PARTNER); }
       if (j + LEAD - 1 < ntiles) { load_v(j + LEAD - 1, 0); load_v(j + LEAD - 1, PARTNER); }
     };
@@ -710,26 +739,68 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
 #endif
     if constexpr (VECMAX) {
       // FP8 P.V: the matrix phase is nothing but MFMAs and their LDS reads (P.V of the previous tile, Q.K^T of the
-      // next); the row maximum, the probabilities and the tile requests all belong to the vector phase, which
-      // is the shorter one.  Group 1, whose vector phase is the even one, issues the requests.
+      // next); the row maximum and the probabilities belong to the vector phase, which is the longer one.  Group 0
+      // issues the tile requests of the period, for both wavefronts of each SIMD pair, after its last Q.K^T MFMA: a
+      // request holds up the wavefront that issues it for 40-50 ns (in-kernel timers; a burst, the same requests
+      // spread over the phase, shared between the groups or staggered by SIMD all cost the same per request), and
+      // the end of group 0's matrix phase is where a wavefront would otherwise wait at the barrier for group 1's
+      // softmax (SAGE_REQ_GROUP=1 puts them at the end of group 1's vector phase instead: 1-3 % slower).
+#if SAGE_REQ_GROUP == 0
       if (grp == 0) {
         for (int j = 0; j <= ntiles; j++) {
-          even_barrier(j, j == 0 ? first_in_flight : 0);
+          SAGE_PH(3);
+          even_barrier(j, issuer_in_flight(j));
+          SAGE_PH(0);
+          if (j == 0) first_value_tile();   // V(0) has one period only: ahead of the first Q.K^T, not after it
           if (j >= 1 && j - 1 < wnt) pv(j - 1);
           if (j < wnt) qk(j);
+          request_tiles(j, false);
+          SAGE_PH(1);
           odd_barrier();
+          SAGE_PH(2);
           if (j < wnt) { rowmax(j); softmax(j); }
         }
       } else {
         for (int j = 0; j <= ntiles; j++) {
-          even_barrier(j, issuer_in_flight(j));
+          SAGE_PH(3);
+          even_barrier(j, j == 0 ? first_in_flight : 0);
+          SAGE_PH(0);
           if (j >= 1 && j - 1 < wnt) { rowmax(j - 1); softmax(j - 1); }
-          request_tiles(j);
+          SAGE_PH(1);
           odd_barrier();
+          SAGE_PH(2);
           if (j >= 1 && j - 1 < wnt) pv(j - 1);
           if (j < wnt) qk(j);
         }
       }
+#else
+      if (grp == 0) {
+        for (int j = 0; j <= ntiles; j++) {
+          SAGE_PH(3);
+          even_barrier(j, j == 0 ? first_in_flight : 0);
+          SAGE_PH(0);
+          if (j >= 1 && j - 1 < wnt) pv(j - 1);
+          if (j < wnt) qk(j);
+          SAGE_PH(1);
+          odd_barrier();
+          SAGE_PH(2);
+          if (j < wnt) { rowmax(j); softmax(j); }
+        }
+      } else {
+        for (int j = 0; j <= ntiles; j++) {
+          SAGE_PH(3);
+          even_barrier(j, issuer_in_flight(j));
+          SAGE_PH(0);
+          if (j >= 1 && j - 1 < wnt) { rowmax(j - 1); softmax(j - 1); }
+          request_tiles(j);
+          SAGE_PH(1);
+          odd_barrier();
+          SAGE_PH(2);
+          if (j >= 1 && j - 1 < wnt) pv(j - 1);
+          if (j < wnt) qk(j);
+        }
+      }
+#endif
     } else if (grp == 0) {
       // FP16 P.V.  The even phase is as long as group 1's softmax, which must not start late: all tile loads of
       // the period are issued here, by the group whose matrix phase has slack, after its P.V.
@@ -758,8 +829,7 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
   if constexpr (MSUM) lsum = osum[0];
   else lsum = xchg32_sum(lsum);
   const float den = RSUM ? osum[0] : lsum;
-  const bool live = den > 0.f;   // a row with no visible key (or no keys at all) yields zeros
-  const float inv = live ? 1.0f / den : 0.f;
+  const float inv = den > 0.f ? 1.0f / den : 0.f;   // a row with no visible key yields zeros
   if (my_row < Lq) {
     if (a.lse && h == 0) {
       // lse_offset: what K smoothing removed from every logit of this row (q . k_mean, base-2 units)
@@ -795,8 +865,7 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
 #pragma unroll
           for (int i = 0; i < 4; i++) {
             f[i] = o[dt][4 * q4 + i] * inv;
-            // (the V scales are not read for a dead row: with no keys at all nothing ever wrote them)
-            if constexpr (PV == 1) f[i] = live ? f[i] * vs_lds[d + i] : 0.f;
+            if constexpr (PV == 1) f[i] *= vs_lds[d + i];
           }
           u16 hv[4];
 #pragma unroll
@@ -828,6 +897,11 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
     for (int i = 0; i < 7; i++) atomicAdd(&g_tile_timing[cls * 8 + i], (unsigned long long)(sage_ts[i + 1] - sage_ts[i]));
     atomicAdd(&g_tile_timing[cls * 8 + 7], 1ull);
     if (w == 0) atomicAdd(&g_tile_timing[24], (unsigned long long)ntiles);
+    if (w == 1 || w == NW - 2) {   // one wavefront of each group
+      const int g = (w >> GSH) & 1;
+      for (int i = 0; i < 4; i++) atomicAdd(&g_tile_timing[32 + 4 * g + i], (unsigned long long)ph_sum[i]);
+      atomicAdd(&g_tile_timing[40 + g], (unsigned long long)ph_n);
+    }
   }
 #endif
 }
@@ -839,14 +913,14 @@ static hipError_t launch_one(const AttnArgs& a, int grid, hipStream_t st) {
   auto kern = attn_kernel<D, NW, BN, PV, CAUSAL, MSUM, MASK, KSUB, QF>;
   // More than 64 KB of dynamic LDS has to be allowed once per kernel and device.
   constexpr int kMaxDevices = 64;
-  static bool attr_done[kMaxDevices] = {};
+  static std::atomic<bool> attr_done[kMaxDevices] = {};   // (two host threads may make the first call at once: setting it twice is harmless)
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return e;
-  if (dev < 0 || dev >= kMaxDevices || !attr_done[dev]) {
+  if (dev < 0 || dev >= kMaxDevices || !attr_done[dev].load(std::memory_order_acquire)) {
     e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return e;
-    if (dev >= 0 && dev < kMaxDevices) attr_done[dev] = true;
+    if (dev >= 0 && dev < kMaxDevices) attr_done[dev].store(true, std::memory_order_release);
   }
   kern<<<dim3(grid), dim3(NW * 64), smem, st>>>(a);
   return hipGetLastError();

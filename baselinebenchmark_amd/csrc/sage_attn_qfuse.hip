@@ -17,9 +17,9 @@ hipError_t launch_attn_qfused(const AttnArgs& a, int D, int pv, bool causal, int
 
 #ifdef SAGE_TIMING
 // Timing build only: copies the interval sums of the kernels of this translation unit (the ones the one-call
-// pipeline runs) to `out` (32 values) and clears them.  Synchronises the device.
+// pipeline runs) to `out` (48 values) and clears them.  Synchronises the device.
 extern "C" int sage_tile_timing(unsigned long long* out) {
-  static const unsigned long long zero[32] = {};
+  static const unsigned long long zero[48] = {};
   if (hipDeviceSynchronize() != hipSuccess) return -1;
   if (hipMemcpyFromSymbol(out, HIP_SYMBOL(sage::g_tile_timing), sizeof(zero)) != hipSuccess) return -1;
   return hipMemcpyToSymbol(HIP_SYMBOL(sage::g_tile_timing), zero, sizeof(zero)) == hipSuccess ? 0 : -1;
