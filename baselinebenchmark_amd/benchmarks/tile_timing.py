@@ -56,6 +56,7 @@ def measure(B, H, S, D, causal, dtype=torch.bfloat16, pv_mode="fp8", blkq=64, bl
     for g in (0, 1):
         n = max(d[40 + g], 1)
         rows[f"group {g} phases"] = [d[32 + 4 * g + k] * TICK_NS / n for k in range(4)]
+    rows["request issue"] = [d[42] * TICK_NS / max(d[43], 1)]
     return rows, tiles
 
 
@@ -70,6 +71,9 @@ def main():
         rows, tiles = measure(B, H, S, D, bool(int(causal)))
         print(f"B{B} H{H} S{S} D{D} causal={bool(int(causal))}: {tiles:.1f} K tiles per workgroup", flush=True)
         for name, vals in rows.items():
+            if len(vals) == 1:
+                print(f"  {name:17s} {vals[0]:.0f} ns per period for the wavefront that issues the tile requests", flush=True)
+                continue
             if len(vals) == 4:
                 print(f"  {name:17s} per period {sum(vals):6.0f} ns | first phase {vals[0]:.0f}, odd barrier {vals[1]:.0f}, "
                       f"second phase {vals[2]:.0f}, even barrier {vals[3]:.0f}", flush=True)

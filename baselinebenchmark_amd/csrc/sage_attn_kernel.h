@@ -129,7 +129,8 @@ constexpr int attn_lds_bytes() { return attn_tile_lds_bytes<D, NW, BN, PV, CAUSA
 // [3][0] = tiles.  SAGE_T(k, x) pins stamp k after the computation of x.
 // Also, in the main loop of the FP8 kernels, four stamps per period (after the even barrier, before and after the odd
 // barrier, at the end of the period) are summed per group: [32 + 4 g + k] = ticks from stamp k to the next one (k = 0:
-// first phase of the period, 1: wait at the odd barrier, 2: second phase, 3: wait at the even barrier), [40 + g] = periods.
+// first phase of the period, 1: wait at the odd barrier, 2: second phase, 3: wait at the even barrier), [40 + g] = periods;
+// [42] / [43] = ticks per period that the issuing wavefront spends on the tile requests.
 #ifdef SAGE_TIMING
 static __device__ unsigned long long g_tile_timing[48];
 #define SAGE_PH(k) do { const long long t_ = __builtin_amdgcn_s_memrealtime(); if (ph_last) ph_sum[((k) + 3) & 3] += t_ - ph_last; ph_last = t_; if ((k) == 0) ph_n++; } while (0)
@@ -172,8 +173,8 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
 #ifdef SAGE_TIMING
   long long sage_ts[8];
   for (int i = 0; i < 8; i++) sage_ts[i] = __builtin_amdgcn_s_memrealtime();
-  long long ph_last = 0, ph_sum[4] = {0, 0, 0, 0};
-  int ph_n = 0;
+  long long ph_last = 0, ph_sum[4] = {0, 0, 0, 0}, rq_sum = 0;
+  int ph_n = 0, rq_n = 0;
 #endif
   const int tid = threadIdx.x, lane = tid & 63;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);  // wavefront index: uniform, keep it scalar
@@ -725,9 +726,17 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
     // period 0 and the requests of the last period may still be in flight at a barrier.
     auto first_value_tile = [&]() { load_v(0, 0); load_v(0, PARTNER); };
     auto request_tiles = [&](int j, bool with_first_value = true) {
+#ifdef SAGE_TIMING
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      const long long rq0 = __builtin_amdgcn_s_memrealtime();
+#endif
       if (LEAD == 2 && j == 0 && with_first_value) first_value_tile();
       if (j + LEAD < ntiles) { load_k(j + LEAD, 0); load_k(j + LEAD, PARTNER); }
       if (j + LEAD - 1 < ntiles) { load_v(j + LEAD - 1, 0); load_v(j + LEAD - 1, PARTNER); }
+#ifdef SAGE_TIMING
+      rq_sum += __builtin_amdgcn_s_memrealtime() - rq0;   // ticks this wavefront spent issuing the requests of a period
+      rq_n++;
+#endif
     };
     auto issuer_in_flight = [&](int j) {
       return j == 0 ? first_in_flight : LEAD == 1 ? 0 : (j + 1 < ntiles ? NK : 0) + (j < ntiles ? NV : 0);
@@ -901,6 +910,8 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
       const int g = (w >> GSH) & 1;
       for (int i = 0; i < 4; i++) atomicAdd(&g_tile_timing[32 + 4 * g + i], (unsigned long long)ph_sum[i]);
       atomicAdd(&g_tile_timing[40 + g], (unsigned long long)ph_n);
+      atomicAdd(&g_tile_timing[42], (unsigned long long)rq_sum);   // [42] / [43]: ticks per period spent issuing the tile requests
+      atomicAdd(&g_tile_timing[43], (unsigned long long)rq_n);
     }
   }
 #endif

@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Headline benchmark: effective attention TOPS of the SageAttention forward path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c0|c1|c2|c3|c4|all] [--no-cpu-baseline]
 
 A step is one full pass of the hot path over the workload, inputs already resident in HBM:
 K mean -> INT8 quantise K and Q -> FP8/FP16 V panels -> fused attention (one `sageattn` call).
@@ -15,7 +15,6 @@ from __future__ import annotations
 import argparse
 import json
 import os
-import statistics
 import sys
 import time
 
@@ -29,10 +28,36 @@ PEAK_INT8_FP8 = 5033.2   # MI355X dense INT8 / FP8 MFMA peak, TOP/s (256 CUs x 2
 PEAK_FP16 = 2516.6       # dense FP16 MFMA peak, TFLOP/s
 
 
-# HBM-side bytes per launch of the attention kernel, from the committed rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# runs on this same command (profiles/attn_kernel_c2_pmc.md): (1 245 800 + 262 140) counter units x 2.0 (the factor the
-# same counters read for a 512 MiB device copy) x 1 KiB.  Measured for config 2 only.
-TRAFFIC_BYTES = {"c2": (1245800 + 262140) * 2.0 * 1024}
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "attn_kernel_traffic.json")
+KERNEL_SOURCES = ["sage_attn_kernel.h", "sage_attn.hip", "sage_attn_qfuse.hip", "sage_attn_mask.hip", "sage_common.h", "sage_launch.h"]
+
+
+def kernel_source_digest() -> str:
+    """sha256 over the sources that define the attention kernel: what a committed counter profile is valid for."""
+    import hashlib
+    h = hashlib.sha256()
+    for name in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, "baselinebenchmark_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()
+
+
+def measured_traffic(workload: str):
+    """HBM-side bytes per launch of the attention kernel from the committed rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+    summary (profiles/attn_kernel_traffic.json, written by `python -m baselinebenchmark_amd.benchmarks.traffic_profile`
+    from the counter runs), valid only for the kernel sources it was measured on.  Returns (bytes or None, note)."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            doc = json.load(f)
+    except (OSError, ValueError) as exc:
+        return None, f"no committed counter profile ({exc.__class__.__name__})"
+    if doc.get("kernel_source_sha256") != kernel_source_digest():
+        return None, "the committed counter profile was measured on other kernel sources (sha256 differs): re-run the --pmc passes"
+    row = doc.get("workloads", {}).get(workload)
+    if row is None:
+        return None, f"no counter profile for workload {workload}"
+    return row["bytes"], (f"FETCH_SIZE {row['fetch_kib']:.0f} KiB x {row['fetch_factor']:.2f} + WRITE_SIZE {row['write_kib']:.0f} KiB x "
+                          f"{row['write_factor']:.2f} per launch (factors from a 512 MiB device copy in the same runs)")
 
 
 def blended_peak(pv: str) -> float:
@@ -44,31 +69,52 @@ def blended_peak(pv: str) -> float:
 
 def time_attention_kernel(sa, S, w, iters: int):
     """Average duration of the fused attention kernel alone, HIP events on the launch stream: the variant
-    the one-call pipeline runs (K and V pre-quantised, Q quantised in the kernel's prologue).  Returns
-    milliseconds per launch."""
+    the one-call pipeline runs (K and V pre-quantised, Q quantised in the kernel's prologue), for fixed-length
+    and packed workloads alike.  Returns milliseconds per launch."""
     import ctypes
     from baselinebenchmark_amd._cabi import check, lib
     kw = w.kwargs
     layout = w.layout
-    if w.cu_seqlens is not None:
-        return None
     q, k, v = w.q, w.k, w.v
-    km = sa.k_mean(k, layout)
-    qi, qs, ki, ks = sa.per_block_int8(q, k, km=km, BLKQ=kw["BLKQ"], BLKK=kw["BLKK"], tensor_layout=layout)
-    panels, vs = sa.prepare_v(v, layout, kw["pv_mode"])
-    out = torch.empty_like(q)
-    B, Hq, Sq, D, qsb, qsh, qsn = S._layout(qi, layout)
-    _, Hkv, Skv, _, ksb, ksh, ksn = S._layout(ki, layout)
-    _, _, _, _, osb, osh, osn = S._layout(out, layout)
     pv = S._pv(kw["pv_mode"])
+    out = torch.empty_like(q)
     stream = torch.cuda.current_stream()
+    st = ctypes.c_void_p(stream.cuda_stream)
+    if w.cu_seqlens is None:
+        km = sa.k_mean(k, layout)
+        _, _, ki, ks = sa.per_block_int8(q, k, km=km, BLKQ=kw["BLKQ"], BLKK=kw["BLKK"], tensor_layout=layout)
+        panels, vs = sa.prepare_v(v, layout, kw["pv_mode"])
+        B, Hq, Sq, D, qsb, qsh, qsn = S._layout(q, layout)
+        _, Hkv, Skv, _, ksb, ksh, ksn = S._layout(ki, layout)
+        _, _, _, _, osb, osh, osn = S._layout(out, layout)
+        args = (B, Hq, Hkv, Sq, Skv, D, qsb, qsh, qsn, ksb, ksh, ksn, osb, osh, osn, kw["BLKQ"], kw["BLKK"], int(w.causal), pv,
+                S._dt(q.dtype), None, None, None, 0, 0, 0, st)
+    else:
+        # packed batch: the same pieces through the C ABI -- plan, K mean per sequence, INT8 K, V panels
+        cu, nseq, L = w.cu_seqlens, w.cu_seqlens.numel() - 1, w.max_seqlen
+        Tq, Hq, D = q.shape
+        Tk, Hkv, _ = k.shape
+        km = torch.empty((nseq, Hkv, D), device=q.device, dtype=k.dtype)
+        nb = lib().sage_k_mean_workspace_bytes(nseq, Hkv, L, D)
+        ws = torch.empty(max(nb, 8), device=q.device, dtype=torch.uint8)
+        check(lib().sage_k_mean(S._ptr(k), S._ptr(km), S._ptr(ws), nb, nseq, Hkv, L, D, 0, k.stride(1), k.stride(0), S._dt(k.dtype),
+                                S._ptr(cu), st))
+        _, _, ki, ks, plan, offs = sa.per_block_int8_varlen(q, k, cu, cu, L, L, km=km, BLKQ=kw["BLKQ"], BLKK=kw["BLKK"])
+        plan, offs = sa.varlen_plan(cu, cu, Tq, kw["BLKQ"], kw["BLKK"], is_causal=w.causal)   # (tile order for this mask)
+        panel_sh = Tk // 128 + nseq
+        panels = torch.zeros(Hkv * panel_sh * 128 * D * (1 if pv else 2), device=q.device, dtype=torch.uint8)
+        vs = torch.empty((nseq, Hkv, D), device=q.device, dtype=torch.float32) if pv else None
+        nb = lib().sage_prep_v_workspace_bytes(nseq, Hkv, L, D, pv)
+        ws = torch.empty(max(nb, 8), device=q.device, dtype=torch.uint8)
+        check(lib().sage_prep_v(S._ptr(v), S._ptr(panels), S._ptr(vs), S._ptr(ws), nb, nseq, Hkv, L, D, 0, v.stride(1), v.stride(0),
+                                S._dt(v.dtype), pv, S._ptr(cu), ctypes.c_void_p(plan.data_ptr() + 4 * offs[2]), panel_sh, st))
+        args = (nseq, Hq, Hkv, L, L, D, 0, q.stride(1), q.stride(0), 0, ki.stride(1), ki.stride(0), 0, out.stride(1), out.stride(0),
+                kw["BLKQ"], kw["BLKK"], int(w.causal), pv, S._dt(q.dtype), S._ptr(cu), S._ptr(cu), S._ptr(plan), Tq,
+                ks.shape[1], panel_sh, st)
 
     def launch():
         check(lib().sage_attn_fwd_qfused(S._ptr(q), S._dt(q.dtype), float(D ** -0.5), S._ptr(ki), S._ptr(panels), S._ptr(ks),
-                                         S._ptr(vs), S._ptr(out), None,
-                                         B, Hq, Hkv, Sq, Skv, D, qsb, qsh, qsn, ksb, ksh, ksn, osb, osh, osn,
-                                         kw["BLKQ"], kw["BLKK"], int(w.causal), pv, S._dt(q.dtype), None, None, None, 0, 0, 0,
-                                         ctypes.c_void_p(stream.cuda_stream)))
+                                         S._ptr(vs), S._ptr(out), None, *args))
     for _ in range(3):
         launch()
     stream.synchronize()
@@ -78,7 +124,7 @@ def time_attention_kernel(sa, S, w, iters: int):
         launch()
     e1.record(stream)
     e1.synchronize()
-    return e0.elapsed_time(e1) / iters
+    return e0.elapsed_time(e1) / iters, out
 
 
 def cpu_baseline(name: str, budget_s: float = 20.0):
@@ -106,6 +152,51 @@ def cpu_baseline(name: str, budget_s: float = 20.0):
     }
 
 
+def run_workload(name: str, args, sa, S, workloads) -> dict:
+    w = workloads.make(name, device="cuda")
+    if w.cu_seqlens is None:
+        def step():
+            return sa.sageattn(w.q, w.k, w.v, **w.kwargs)
+    else:
+        def step():
+            return sa.sageattn(w.q, w.k, w.v, cu_seqlens_q=w.cu_seqlens, cu_seqlens_k=w.cu_seqlens, max_seqlen_q=w.max_seqlen,
+                               max_seqlen_k=w.max_seqlen, **w.kwargs)
+
+    for _ in range(args.warmup):
+        ref = step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    value = w.ops / (ms * 1e-3) / 1e12
+
+    pv = w.kwargs["pv_mode"]
+    peak = blended_peak(pv)
+    kms, kout = time_attention_kernel(sa, S, w, max(args.steps, 10))
+    if args.warmup > 0 and not torch.equal(kout, ref):
+        raise RuntimeError("the separately launched attention kernel does not reproduce the one-call result")
+    achieved = w.ops / (kms * 1e-3) / 1e12
+    traffic, traffic_note = measured_traffic(name)
+    roofline = {"bound": "mfma", "achieved": round(achieved, 1), "peak": round(peak, 1), "unit": "TFLOP/s",
+                "frac": round(achieved / peak, 4), "traffic": traffic, "traffic_note": traffic_note,
+                "kernel": "sage::attn_kernel", "kernel_ms": round(kms, 4),
+                "note": "algorithmic ops = 4*B*Hq*Sq*Skv*D*(1/2 causal) per launch / HIP-event average launch time"}
+    out = {
+        "metric": METRIC, "value": round(value, 1), "unit": "TOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int8 QK / " + ("fp8-e4m3 PV" if pv == "fp8" else "fp16 PV") + " / fp32 softmax+accumulate",
+        "data": "synthetic",
+        "config": {"workload": w.desc, "step": "K mean + INT8 quantise Q,K + V panels + fused attention (sageattn)",
+                   "effective_ops": w.ops, "frac_of_mfma_peak_end_to_end": round(value / peak, 4)},
+        "roofline": roofline,
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(name if name != "c4" else "c2", args.cpu_seconds)
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -113,7 +204,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=30,
                     help="untimed steps before the timed ones; the first dozen steps after idle run up to 30 %% slower "
                          "while the GPU clocks ramp, so the default covers that transient")
-    ap.add_argument("--workload", default="c2", choices=["c0", "c1", "c2", "c3", "c4"])
+    ap.add_argument("--workload", default="c2", choices=["c0", "c1", "c2", "c3", "c4", "all"],
+                    help="BASELINE configuration; 'all' prints one JSON line per configuration (the CPU baseline only on c2)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=20.0)
     ap.add_argument("--copy-calibration", action="store_true",
@@ -130,53 +222,22 @@ def main():
     from baselinebenchmark_amd import workloads
 
     torch.cuda.set_device(0)
-    w = workloads.make(args.workload, device="cuda")
-
-    if w.cu_seqlens is None:
-        def step():
-            return sa.sageattn(w.q, w.k, w.v, **w.kwargs)
-    else:
-        def step():
-            return sa.sageattn_varlen(w.q, w.k, w.v, w.cu_seqlens, w.cu_seqlens, w.max_seqlen, w.max_seqlen, **w.kwargs)
-
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    ms = (time.perf_counter() - t0) * 1e3 / args.steps
-    value = w.ops / (ms * 1e-3) / 1e12
-
-    pv = w.kwargs["pv_mode"]
-    peak = blended_peak(pv)
-    kms = time_attention_kernel(sa, S, w, max(args.steps, 10))
-    roofline = None
-    if kms is not None:
-        achieved = w.ops / (kms * 1e-3) / 1e12
-        roofline = {"bound": "mfma", "achieved": round(achieved, 1), "peak": round(peak, 1), "unit": "TFLOP/s",
-                    "frac": round(achieved / peak, 4), "traffic": TRAFFIC_BYTES.get(args.workload),
-                    "kernel": "sage::attn_kernel", "kernel_ms": round(kms, 4),
-                    "note": "algorithmic ops = 4*B*Hq*Sq*Skv*D*(1/2 causal) per launch / HIP-event average launch time"}
-    out = {
-        "metric": METRIC, "value": round(value, 1), "unit": "TOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "int8 QK / " + ("fp8-e4m3 PV" if pv == "fp8" else "fp16 PV") + " / fp32 softmax+accumulate",
-        "data": "synthetic",
-        "config": {"workload": w.desc, "step": "K mean + INT8 quantise Q,K + V panels + fused attention (sageattn)",
-                   "effective_ops": w.ops, "frac_of_mfma_peak_end_to_end": round(value / peak, 4)},
-        "roofline": roofline,
-    }
+    names = ["c0", "c1", "c2", "c3", "c4"] if args.workload == "all" else [args.workload]
+    for name in names:
+        if args.workload == "all" and name != "c2":
+            saved, args.no_cpu_baseline = args.no_cpu_baseline, True
+            out = run_workload(name, args, sa, S, workloads)
+            args.no_cpu_baseline = saved
+        else:
+            out = run_workload(name, args, sa, S, workloads)
+        print(json.dumps(out), flush=True)
+        torch.cuda.empty_cache()
     if args.copy_calibration:
         x = torch.empty(128 * 1024 * 1024, device="cuda", dtype=torch.int32)
         y = torch.empty_like(x)
         for _ in range(3):
             y.copy_(x)
         torch.cuda.synchronize()
-    if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(args.workload if args.workload != "c4" else "c2", args.cpu_seconds)
-    print(json.dumps(out))
 
 
 if __name__ == "__main__":

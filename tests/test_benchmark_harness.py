@@ -103,6 +103,9 @@ def test_tile_timing_tool_reports_the_intervals_of_a_workgroup():
     doc = json.loads([l for l in res.stdout.splitlines() if l.startswith("{")][-1])
     assert abs(doc["tiles"] - 17.0) < 1e-6          # 16 q-tiles of 256 rows: 2, 4, ..., 32 K tiles of 128 keys
     for name, vals in doc["rows"].items():
+        if name == "request issue":
+            assert len(vals) == 1 and vals[0] > 0
+            continue
         if name.endswith("phases"):          # main-loop phases per period: two phases and the waits at the two barriers
             assert len(vals) == 4 and all(v >= 0 for v in vals) and vals[0] > 0 and vals[2] > 0, (name, vals)
             continue
