@@ -10,6 +10,11 @@
  * 4 * waves_per_simd wavefronts (1, 2 or 4 per SIMD), `iters` iterations each, on `stream` (a hipStream_t); the
  * caller times the launch.  sage_microbench_units gives the work of one wavefront per iteration: operations (a
  * multiply-add counts 2), bytes, or instructions.  `sink` (device memory) takes grid * 1024 ints.
+ *
+ * sage_coexec: how much the matrix pipe and the vector ALU of a SIMD slow each other down.  Workgroups of eight
+ * wavefronts (two per SIMD): wavefronts 0-3 issue MFMAs (mfma_kind 0 INT8 32x32x32, 1 FP8 32x32x64; 16 per iteration),
+ * wavefronts 4-7 vector instructions (valu_kind 0 v_fma_f32, 1 v_cvt_pk_u8_f32, 2 v_max3_i32, 3 the mix of the FP8
+ * softmax: 64 + 64 + 32 per iteration).  mode 1 runs the MFMA half alone, 2 the vector half alone, 3 both.
  */
 #ifndef SAGE_HW_RATES_H
 #define SAGE_HW_RATES_H
@@ -23,6 +28,7 @@ extern "C" {
 #define HWR_ESIZE (-5)
 double sage_microbench_units(int kind);
 int sage_microbench(int kind, int grid, int waves_per_simd, int iters, void* sink, size_t sink_bytes, void* stream);
+int sage_coexec(int mfma_kind, int valu_kind, int mode, int grid, int iters, void* sink, size_t sink_bytes, void* stream);
 #ifdef __cplusplus
 }
 #endif

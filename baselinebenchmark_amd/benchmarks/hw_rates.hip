@@ -113,6 +113,72 @@ __global__ void __launch_bounds__(1024) microbench_kernel(int* sink, int iters, 
   sink[blockIdx.x * 1024 + threadIdx.x] = result;
 }
 
+// Co-execution of the two pipes of a SIMD: a workgroup of eight wavefronts, two per SIMD; wavefronts 0-3 issue MFMAs
+// (MK 0: v_mfma_i32_32x32x32_i8, 1: v_mfma_f32_32x32x64_f8f6f4, four accumulators in turn), wavefronts 4-7 vector
+// instructions (VK 0: v_fma_f32, 1: v_cvt_pk_u8_f32, 2: v_max3_i32, 3: the mix of the FP8 softmax without v_exp_f32: per
+// 64 scores 64 fma + 64 cvt_pk_u8 + 32 max3).  mode bit 0 / 1 switches each half on: timing a half alone and both together
+// says how much the pipes slow each other down.  Per iteration: 16 MFMAs, or 64 / 64 / 32 / 160 vector instructions.
+template <int MK, int VK>
+__global__ void __launch_bounds__(512) coexec_kernel(int* sink, int iters, int mode, float s, float c) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  int result = 0;
+  if (wave < 4) {
+    if (!(mode & 1)) return;
+    v8i a8 = {lane, 1, 2, 3, 4, 5, 6, 7};
+    v4i a4 = {lane, 1, 2, 3};
+    v16f accf[4] = {};
+    v16i acci[4] = {};
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+      for (int i = 0; i < 16; i++) {
+        if constexpr (MK == 0) acci[i & 3] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a4, a4, acci[i & 3], 0, 0, 0);
+        else accf[i & 3] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a8, a8, accf[i & 3], 0, 0, 0, 0, 0, 0);
+      }
+    }
+    for (int k = 0; k < 4; k++) result ^= MK == 0 ? acci[k][0] : (int)accf[k][0];
+  } else {
+    if (!(mode & 2)) return;
+    float x[16];
+    unsigned pk[4] = {0, 0, 0, 0};
+    int mx[4] = {0, 0, 0, 0};
+    for (int i = 0; i < 16; i++) x[i] = lane * 1e-3f + i * 0.01f;
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+      for (int u = 0; u < 4; u++) {
+        if constexpr (VK == 0 || VK == 3) {
+#pragma unroll
+          for (int i = 0; i < 16; i++) x[i] = __builtin_fmaf(x[i], s, c);
+        }
+        if constexpr (VK == 1 || VK == 3) {
+#pragma unroll
+          for (int i = 0; i < 16; i++) pk[i >> 2] = __builtin_amdgcn_cvt_pk_u8_f32(x[i], i & 3, pk[i >> 2]);
+        }
+        if constexpr (VK == 2 || VK == 3) {
+#pragma unroll
+          for (int i = 0; i < 16; i += 2)
+            mx[(i >> 1) & 3] = max(max(mx[(i >> 1) & 3], __builtin_bit_cast(int, x[i])), __builtin_bit_cast(int, x[i + 1]));
+        }
+        // nothing of an iteration is loop invariant or dead
+#pragma unroll
+        for (int i = 0; i < 4; i++) asm volatile("" : "+v"(pk[i]), "+v"(mx[i]));
+#pragma unroll
+        for (int i = 0; i < 16; i++) asm volatile("" : "+v"(x[i]));
+      }
+    }
+    float r = 0.f;
+    for (int i = 0; i < 16; i++) r += x[i];
+    for (int i = 0; i < 4; i++) result ^= (int)pk[i] ^ mx[i];
+    result ^= (int)r;
+  }
+  sink[blockIdx.x * 1024 + threadIdx.x] = result;
+}
+
+template <int MK, int VK>
+hipError_t launch_coexec(int* sink, int grid, int iters, int mode, hipStream_t st) {
+  coexec_kernel<MK, VK><<<dim3(grid), dim3(512), 0, st>>>(sink, iters, mode, 0.999f, 0.001f);
+  return hipGetLastError();
+}
+
 template <int KIND>
 hipError_t launch_mb(int* sink, int grid, int waves, int iters, hipStream_t st) {
   microbench_kernel<KIND><<<dim3(grid), dim3(waves * 64), 0, st>>>(sink, iters, waves, 0.999f, 0.001f);
@@ -161,6 +227,24 @@ int sage_microbench(int kind, int grid, int waves_per_simd, int iters, void* sin
     case MB_CVT_FP8: e = launch_mb<MB_CVT_FP8>(out, grid, waves, iters, st); break;
     default: e = launch_mb<MB_SOFTMAX_MIX>(out, grid, waves, iters, st); break;
   }
+  return e == hipSuccess ? HWR_OK : HWR_ELAUNCH;
+}
+
+// Co-execution benchmark: `grid` workgroups of eight wavefronts, `iters` iterations; mfma_kind 0 (INT8) or 1 (FP8),
+// valu_kind 0 fma, 1 cvt_pk_u8, 2 max3, 3 the mix; mode 1 = the MFMA wavefronts only, 2 = the vector wavefronts only,
+// 3 = both.  Per iteration a wavefront issues 16 MFMAs, or 64 / 64 / 32 / 160 vector instructions.
+int sage_coexec(int mfma_kind, int valu_kind, int mode, int grid, int iters, void* sink, size_t sink_bytes, void* stream) {
+  using namespace sage;
+  if (mfma_kind < 0 || mfma_kind > 1 || valu_kind < 0 || valu_kind > 3 || mode < 1 || mode > 3) return HWR_EINVAL;
+  if (grid <= 0 || grid > 65535 || iters <= 0 || !sink) return HWR_EINVAL;
+  if (sink_bytes < (size_t)grid * 1024 * sizeof(int)) return HWR_ESIZE;
+  int* out = (int*)sink;
+  hipStream_t st = (hipStream_t)stream;
+  hipError_t e;
+#define SAGE_CX(M, V) launch_coexec<M, V>(out, grid, iters, mode, st)
+  if (mfma_kind == 0) e = valu_kind == 0 ? SAGE_CX(0, 0) : valu_kind == 1 ? SAGE_CX(0, 1) : valu_kind == 2 ? SAGE_CX(0, 2) : SAGE_CX(0, 3);
+  else e = valu_kind == 0 ? SAGE_CX(1, 0) : valu_kind == 1 ? SAGE_CX(1, 1) : valu_kind == 2 ? SAGE_CX(1, 2) : SAGE_CX(1, 3);
+#undef SAGE_CX
   return e == hipSuccess ? HWR_OK : HWR_ELAUNCH;
 }
 

@@ -31,6 +31,8 @@ def lib() -> ctypes.CDLL:
         h.sage_microbench_units.argtypes = [ctypes.c_int]
         h.sage_microbench.restype = ctypes.c_int
         h.sage_microbench.argtypes = [ctypes.c_int] * 4 + [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
+        h.sage_coexec.restype = ctypes.c_int
+        h.sage_coexec.argtypes = [ctypes.c_int] * 5 + [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
         _lib = h
     return _lib
 
@@ -92,13 +94,47 @@ def run(iters_mfma: int = 4000, iters_valu: int = 20000) -> list[dict]:
     return rows
 
 
+COEXEC_MFMA = ["v_mfma_i32_32x32x32_i8", "v_mfma_f32_32x32x64_f8f6f4 (fp8)"]
+COEXEC_VALU = [("v_fma_f32", 64), ("v_cvt_pk_u8_f32", 64), ("v_max3_i32", 32), ("softmax mix: 64 fma + 64 cvt_pk_u8 + 32 max3", 160)]
+
+
+def run_coexec(iters: int = 20000) -> list[dict]:
+    """Two wavefronts per SIMD, one issuing MFMAs and one vector instructions: each half alone, then both.  While both
+    run, each pipe's rate is (its time alone) / (time it needed next to the other); the half that finishes first leaves
+    the other one alone for the rest, which the two-equation estimate below accounts for."""
+    n_cu = torch.cuda.get_device_properties(0).multi_processor_count
+    sink = torch.empty(n_cu * 1024, dtype=torch.int32, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    def timed(mk, vk, mode):
+        def launch():
+            check(lib().sage_coexec(mk, vk, mode, n_cu, iters, sink.data_ptr(), sink.numel() * 4, stream))
+        launch()
+        torch.cuda.synchronize()
+        best = float("inf")
+        for _ in range(3):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(); launch(); e1.record()
+            torch.cuda.synchronize()
+            best = min(best, e0.elapsed_time(e1) * 1e-3)
+        return best
+    rows = []
+    for mk, mname in enumerate(COEXEC_MFMA):
+        for vk, (vname, vinstr) in enumerate(COEXEC_VALU):
+            tm, tv, tb = timed(mk, vk, 1), timed(mk, vk, 2), timed(mk, vk, 3)
+            rows.append({"mfma": mname, "valu": vname, "mfma_alone_s": tm, "valu_alone_s": tv, "both_s": tb,
+                         "ns_per_mfma": tm / (16 * iters) * 1e9, "ns_per_valu_instruction": tv / (vinstr * iters) * 1e9,
+                         "overlap": (tm + tv - tb) / min(tm, tv)})
+    return rows
+
+
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(description=__doc__)
     ap.add_argument("--json", action="store_true", help="print one JSON document instead of the table")
     args = ap.parse_args(argv)
     rows = run()
+    co = run_coexec()
     if args.json:
-        print(json.dumps(rows))
+        print(json.dumps({"rates": rows, "coexecution": co}))
         return 0
     print(f"{'benchmark':58s} waves/SIMD  result")
     for r in rows:
@@ -109,6 +145,12 @@ def main(argv=None) -> int:
         else:
             res = f"{r['ns_per_instruction_per_SIMD']:7.2f} ns per wavefront instruction per SIMD"
         print(f"{r['name']:58s} {r['waves_per_simd']:^10d}  {res}")
+    print("\nco-execution on one SIMD (one wavefront issues MFMAs, the other vector instructions); overlap = share of the shorter"
+          " half's time that is hidden when both run")
+    for r in co:
+        print(f"{r['mfma']:34s} + {r['valu']:46s} alone {r['mfma_alone_s'] * 1e3:6.3f} / {r['valu_alone_s'] * 1e3:6.3f} ms "
+              f"({r['ns_per_mfma']:.1f} ns per MFMA, {r['ns_per_valu_instruction']:.2f} ns per vector instruction), both "
+              f"{r['both_s'] * 1e3:6.3f} ms, overlap {100 * r['overlap']:.0f} %")
     return 0
 
 

@@ -57,6 +57,7 @@ def measure(B, H, S, D, causal, dtype=torch.bfloat16, pv_mode="fp8", blkq=64, bl
         n = max(d[40 + g], 1)
         rows[f"group {g} phases"] = [d[32 + 4 * g + k] * TICK_NS / n for k in range(4)]
     rows["request issue"] = [d[42] * TICK_NS / max(d[43], 1)]
+    rows["raw Q wait"] = [d[44] * TICK_NS / max(d[45], 1)]
     return rows, tiles
 
 
@@ -71,6 +72,9 @@ def main():
         rows, tiles = measure(B, H, S, D, bool(int(causal)))
         print(f"B{B} H{H} S{S} D{D} causal={bool(int(causal))}: {tiles:.1f} K tiles per workgroup", flush=True)
         for name, vals in rows.items():
+            if name == "raw Q wait":
+                print(f"  {name:17s} {vals[0]:.0f} ns from a wavefront's last prologue request to the arrival of its raw Q rows", flush=True)
+                continue
             if len(vals) == 1:
                 print(f"  {name:17s} {vals[0]:.0f} ns per period for the wavefront that issues the tile requests", flush=True)
                 continue

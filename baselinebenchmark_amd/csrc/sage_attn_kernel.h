@@ -130,7 +130,8 @@ constexpr int attn_lds_bytes() { return attn_tile_lds_bytes<D, NW, BN, PV, CAUSA
 // Also, in the main loop of the FP8 kernels, four stamps per period (after the even barrier, before and after the odd
 // barrier, at the end of the period) are summed per group: [32 + 4 g + k] = ticks from stamp k to the next one (k = 0:
 // first phase of the period, 1: wait at the odd barrier, 2: second phase, 3: wait at the even barrier), [40 + g] = periods;
-// [42] / [43] = ticks per period that the issuing wavefront spends on the tile requests.
+// [42] / [43] = ticks per period that the issuing wavefront spends on the tile requests; [44] / [45] = ticks a wavefront
+// of the kernels that quantise their own Q waits, after its last prologue request, for the raw rows to arrive.
 #ifdef SAGE_TIMING
 static __device__ unsigned long long g_tile_timing[48];
 #define SAGE_PH(k) do { const long long t_ = __builtin_amdgcn_s_memrealtime(); if (ph_last) ph_sum[((k) + 3) & 3] += t_ - ph_last; ph_last = t_; if ((k) == 0) ph_n++; } while (0)
@@ -173,7 +174,7 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
 #ifdef SAGE_TIMING
   long long sage_ts[8];
   for (int i = 0; i < 8; i++) sage_ts[i] = __builtin_amdgcn_s_memrealtime();
-  long long ph_last = 0, ph_sum[4] = {0, 0, 0, 0}, rq_sum = 0;
+  long long ph_last = 0, ph_sum[4] = {0, 0, 0, 0}, rq_sum = 0, q_wait = 0;
   int ph_n = 0, rq_n = 0;
 #endif
   const int tid = threadIdx.x, lane = tid & 63;
@@ -334,7 +335,13 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
         const int u = (lane % QUPR) ^ (r & (QUPR - 1));
         dma16(qrsrc, min(row0 + r, Lq - 1) * (int)a.q_sn * 2 + 16 * u, 0, qstage + i * 1024);
       }
+#ifdef SAGE_TIMING
+      const long long q_issued = __builtin_amdgcn_s_memrealtime();
+#endif
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#ifdef SAGE_TIMING
+      q_wait = __builtin_amdgcn_s_memrealtime() - q_issued;   // from the last request of the prologue to the arrival of everything
+#endif
     }
     float x[KS][16];
     float amax = 0.f;
@@ -912,6 +919,8 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
       atomicAdd(&g_tile_timing[40 + g], (unsigned long long)ph_n);
       atomicAdd(&g_tile_timing[42], (unsigned long long)rq_sum);   // [42] / [43]: ticks per period spent issuing the tile requests
       atomicAdd(&g_tile_timing[43], (unsigned long long)rq_n);
+      atomicAdd(&g_tile_timing[44], (unsigned long long)q_wait);   // [44] / [45]: ticks a wavefront waits for its raw Q rows (and the first K tile)
+      atomicAdd(&g_tile_timing[45], 1ull);
     }
   }
 #endif

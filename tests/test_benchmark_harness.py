@@ -82,6 +82,13 @@ def test_hw_rate_microbenchmarks_run_and_are_plausible():
             best[r["kind"]] = max(best.get(r["kind"], 0.0), r["chip_TOPS"])
     assert best[0] > 2500 and best[1] > 2500, best
     assert best[3] <= best[0] * 1.05 and best[4] <= best[1] * 1.05, best   # feeding from LDS never beats registers
+    # co-execution: running the MFMA wavefront and the vector wavefront of a SIMD together takes at least as long as the
+    # longer half alone and no longer than both in a row (a little slack for launch overhead on these short runs)
+    co = hw_rates.run_coexec(iters=2000)
+    assert len(co) == len(hw_rates.COEXEC_MFMA) * len(hw_rates.COEXEC_VALU)
+    for r in co:
+        assert r["both_s"] > 0.9 * max(r["mfma_alone_s"], r["valu_alone_s"]), r
+        assert r["both_s"] < 1.15 * (r["mfma_alone_s"] + r["valu_alone_s"]), r
 
 
 @pytest.mark.gpu
@@ -105,6 +112,9 @@ def test_tile_timing_tool_reports_the_intervals_of_a_workgroup():
     for name, vals in doc["rows"].items():
         if name == "request issue":
             assert len(vals) == 1 and vals[0] > 0
+            continue
+        if name == "raw Q wait":               # prologue: last request issued -> raw Q rows (and the first K tile) in LDS
+            assert len(vals) == 1 and 0 < vals[0] < 1.0e5
             continue
         if name.endswith("phases"):          # main-loop phases per period: two phases and the waits at the two barriers
             assert len(vals) == 4 and all(v >= 0 for v in vals) and vals[0] > 0 and vals[2] > 0, (name, vals)
