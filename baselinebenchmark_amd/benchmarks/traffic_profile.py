@@ -6,8 +6,9 @@
     python -m baselinebenchmark_amd.benchmarks.traffic_profile --runs <dir> --workloads c2 [c1 c3 c4 ...]
 
 For every workload it averages FETCH_SIZE and WRITE_SIZE (KiB per dispatch, summed over the counter's instances) over
-the launches of sage::attn_kernel, scales each by what the same counter reads for the 512 MiB device-to-device copy
-that `--copy-calibration` appends to the run (a kernel of known traffic: 524 288 KiB read, 524 288 KiB written), and
+the launches of sage::attn_kernel, scales each by what the same counter reads for the 512 MiB device-to-device copies
+that `--copy-calibration` appends to the run (`__amd_rocclr_copyBuffer`, a kernel of known traffic: 524 288 KiB read,
+524 288 KiB written; on MI355X FETCH_SIZE reads half of the KiB fetched and WRITE_SIZE all of the KiB written), and
 writes profiles/attn_kernel_traffic.json together with the sha256 of the kernel sources the runs were made on
 (bench.py prints `traffic: null` when the sources have changed since).
 """
@@ -39,9 +40,10 @@ def _counter_means(run_dir: str, counter: str):
             key = (f, r["Dispatch_Id"])
             per_dispatch[key] += float(r["Counter_Value"])
             name = r["Kernel_Name"]
-            kind[key] = "attn" if "attn_kernel" in name else "copy" if ("elementwise_kernel" in name and "copy" in name.lower()) else "other"
+            # the calibration copy of bench.py (same dtype, contiguous) runs as the runtime's own copy kernel
+            kind[key] = "attn" if "attn_kernel" in name else "copy" if "rocclr_copyBuffer" in name else "other"
     attn = [v for k, v in per_dispatch.items() if kind[k] == "attn"]
-    copy = [v for k, v in per_dispatch.items() if kind[k] == "copy"]
+    copy = [v for k, v in per_dispatch.items() if kind[k] == "copy" and v > 1024.0]   # (not the few-byte copies of scalars)
     if not attn or not copy:
         raise SystemExit(f"{run_dir}: {len(attn)} attention launches and {len(copy)} copy launches found for {counter}")
     return sum(attn) / len(attn), sum(copy) / len(copy), len(attn)

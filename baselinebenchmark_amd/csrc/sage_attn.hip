@@ -66,7 +66,46 @@ __global__ void __launch_bounds__(1024) varlen_plan_kernel(const int32_t* cu_q, 
     if (tid == 1023) plan[L.ntiles] = before + incl;
   }
   __syncthreads();
-  // pass 2: place tiles, most expensive bins first
+  // pass 2: place tiles.  Few sequences (the usual case): cost TIERS of kTierCost cost units (eight causal q-tiles of
+  // 256 rows when the unit is 64 keys), most expensive tier first;
+  // inside a tier sequence by sequence, and inside a sequence the heavier q-tiles first.  Consecutive entries of the
+  // list run at the same time (eight of them per XCD when an XCD holds one KV head), and q-tiles of one sequence
+  // walk the same K/V tiles from tile 0 on at about the same pace: one fetches a tile into the XCD's L2, the others
+  // hit it there.  Ordered by cost alone, neighbours in the list belong to different sequences and share nothing.
+  // The q-tiles of a sequence that fall into one tier are a contiguous range (cost does not decrease with the tile
+  // index), so a tile's place is the tier's fill level plus its distance from the heaviest tile of that range.
+  constexpr int kTierCost = 32, kTiers = kCostBins / kTierCost, kMaxTieredSeqs = 64;
+  if (nseq <= kMaxTieredSeqs) {
+    __shared__ int tier_fill[kTiers], tier_max[kTiers], tier_cnt[kTiers];
+    if (tid == 0) {
+      int before = 0;
+      for (int t = kTiers - 1; t >= 0; t--) {
+        tier_fill[t] = before;
+        for (int c = 0; c < kTierCost; c++) before += hist[t * kTierCost + c];
+      }
+    }
+    for (int i = 0; i < nseq; i++) {
+      const int lq = cu_q[i + 1] - cu_q[i], lk = cu_k[i + 1] - cu_k[i];
+      const int nqt = (lq + bm - 1) / bm;
+      for (int t = tid; t < kTiers; t += blockDim.x) { tier_max[t] = -1; tier_cnt[t] = 0; }
+      __syncthreads();
+      for (int qt = tid; qt < nqt; qt += blockDim.x) {
+        const int t = cost_of(lq, lk, qt) / kTierCost;
+        atomicMax(&tier_max[t], qt);
+        atomicAdd(&tier_cnt[t], 1);
+      }
+      __syncthreads();
+      for (int qt = tid; qt < nqt; qt += blockDim.x) {
+        const int t = cost_of(lq, lk, qt) / kTierCost;
+        tiles[tier_fill[t] + tier_max[t] - qt] = (i << 16) | qt;
+      }
+      __syncthreads();
+      for (int t = tid; t < kTiers; t += blockDim.x) tier_fill[t] += tier_cnt[t];
+      __syncthreads();
+    }
+    return;
+  }
+  // Many sequences: most expensive cost bins first, in whatever order the tiles of a bin arrive.
   for (int i = 0; i < nseq; i++) {
     int lq = cu_q[i + 1] - cu_q[i], lk = cu_k[i + 1] - cu_k[i];
     int nqt = (lq + bm - 1) / bm;

@@ -186,7 +186,28 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
   const int G = a.Hq / a.Hkv;
   int rank, s, NG;
   if (packed) { rank = blockIdx.x / a.Hq; s = blockIdx.x % a.Hq; NG = a.Hkv; }
-  else { int U = a.B * a.Hq; rank = blockIdx.x / U; s = blockIdx.x % U; NG = a.B * a.Hkv; }
+  else {
+    const int U = a.B * a.Hq;
+    NG = a.B * a.Hkv;
+#ifndef SAGE_RANK_MAJOR
+    constexpr int TIER = 32;   // compute units of an XCD
+    if ((U & 7) == 0 && (NG & 7) == 0 && a.nqt >= TIER) {
+      // Inside an XCD (workgroup index modulo 8) the compute units take TIER q-tiles of ONE head at a time: the
+      // heaviest TIER q-tiles of its first head, of its second head, ..., then the next TIER of each head, and so on
+      // (a last, smaller tier if TIER does not divide the q-tiles).  The q-tiles of a head walk the same K/V tiles from
+      // tile 0 on at about the same pace, so one of them fetches a tile into the XCD's L2 and the others hit it
+      // there: a quarter to a fifth of the L2 fills of the plain heaviest-first order (where an XCD works on all its
+      // heads at once), and still heavy tiles before light ones.  Short sequences keep the plain order.
+      const int x = blockIdx.x & 7, l = blockIdx.x >> 3, hpx = U >> 3;   // XCD, index inside it, heads per XCD
+      const int nfull = a.nqt / TIER, lfull = nfull * TIER * hpx;
+      int y;
+      if (l < lfull) { const int t = l / (TIER * hpx), rem = l % (TIER * hpx); y = rem / TIER; rank = TIER * t + rem % TIER; }
+      else { const int tl = a.nqt - nfull * TIER, lr = l - lfull; y = lr / tl; rank = nfull * TIER + lr % tl; }
+      s = x + 8 * y;
+    } else
+#endif
+    { rank = blockIdx.x / U; s = blockIdx.x % U; }
+  }
   int gi, g;
   if ((NG & 7) == 0) { int x = s & 7, y = s >> 3; gi = x + 8 * (y / G); g = y % G; }
   else { gi = s / G; g = s % G; }

@@ -48,7 +48,7 @@ def test_varlen_equals_fixed_length_calls_bitwise():
         assert torch.equal(out[sl].cpu(), o[0].cpu()), i
 
 
-def test_plan_orders_tiles_by_decreasing_cost_and_covers_every_tile():
+def test_plan_orders_tiles_by_cost_tier_then_sequence_and_covers_every_tile():
     lens = [512, 4096, 100, 2049, 1, 777]
     cu = torch.tensor(np.concatenate([[0], np.cumsum(lens)]), dtype=torch.int32).to(DEV)
     plan, offs = sa.varlen_plan(cu, cu, int(cu[-1]), 64, 128, is_causal=True)
@@ -60,8 +60,10 @@ def test_plan_orders_tiles_by_decreasing_cost_and_covers_every_tile():
     got = {(int(t) >> 16, int(t) & 0xFFFF) for t in tiles}
     assert got == expect and n == len(expect)
     cost = [min(lens[int(t) >> 16], ((int(t) & 0xFFFF) + 1) * bm) for t in tiles]
-    cost = [(c + 63) // 64 for c in cost]
-    assert cost == sorted(cost, reverse=True)
+    cost = [(c + 63) // 64 for c in cost]            # the scheduler's cost unit: 64 keys
+    # most expensive tier (32 units) first; inside a tier sequence by sequence, inside a sequence heaviest tile first
+    key = [(-(c // 32), int(t) >> 16, -(int(t) & 0xFFFF)) for c, t in zip(cost, tiles)]
+    assert key == sorted(key)
     assert p[offs[2]:offs[2] + 7].tolist() == np.concatenate([[0], np.cumsum([(L + 127) // 128 for L in lens])]).tolist()
 
 
