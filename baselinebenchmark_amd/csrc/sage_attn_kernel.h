@@ -190,20 +190,28 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
     const int U = a.B * a.Hq;
     NG = a.B * a.Hkv;
 #ifndef SAGE_RANK_MAJOR
-    constexpr int TIER = 32;   // compute units of an XCD
-    if ((U & 7) == 0 && (NG & 7) == 0 && a.nqt >= TIER) {
-      // Inside an XCD (workgroup index modulo 8) the compute units take TIER q-tiles of ONE head at a time: the
-      // heaviest TIER q-tiles of its first head, of its second head, ..., then the next TIER of each head, and so on
-      // (a last, smaller tier if TIER does not divide the q-tiles).  The q-tiles of a head walk the same K/V tiles from
-      // tile 0 on at about the same pace, so one of them fetches a tile into the XCD's L2 and the others hit it
-      // there: a quarter to a fifth of the L2 fills of the plain heaviest-first order (where an XCD works on all its
-      // heads at once), and still heavy tiles before light ones.  Short sequences keep the plain order.
+    // (Causal problems with fewer than 16 q-tiles per compute unit keep the plain heaviest-first order: with so few
+    // rounds the balance of the last one matters more than locality -- 5 % on 4 x 32 heads of 4096 rows.)
+    if ((U & 7) == 0 && (NG & 7) == 0 && (!CAUSAL || a.nqt * (U >> 3) >= 512)) {
+      // Inside an XCD (workgroup index modulo 8; 32 compute units) the workgroups that run at the same time take
+      // neighbouring q-tiles of FEW heads: a tier is R consecutive q-tiles (by weight) of each of 32 / R heads.  Tiers go
+      // head group by head group through the heaviest R q-tiles, then through the next R, and so on; R is at most half
+      // the q-tiles of a head (a power of two up to 32), so that the last tiers are light ones and the compute units
+      // finish together.  Long sequences get R = 32: one head at a time.  The q-tiles of a head walk the same K/V
+      // tiles from tile 0 on at about the same pace, so one of them fetches a tile into the XCD's L2 and the others
+      // hit it there (a quarter of the L2 fills of the plain heaviest-first order, where an XCD works on all its heads
+      // at once), and neighbouring q-tiles read neighbouring rows of Q (the raw Q tile arrives in about half the time).
       const int x = blockIdx.x & 7, l = blockIdx.x >> 3, hpx = U >> 3;   // XCD, index inside it, heads per XCD
-      const int nfull = a.nqt / TIER, lfull = nfull * TIER * hpx;
-      int y;
-      if (l < lfull) { const int t = l / (TIER * hpx), rem = l % (TIER * hpx); y = rem / TIER; rank = TIER * t + rem % TIER; }
-      else { const int tl = a.nqt - nfull * TIER, lr = l - lfull; y = lr / tl; rank = nfull * TIER + lr % tl; }
-      s = x + 8 * y;
+      int R = 32;
+      while (R > 1 && 2 * R > a.nqt) R >>= 1;
+      const int Hg = 32 / R;
+      const int nfull = a.nqt / R, lfull = nfull * R * hpx;
+      int t, Rt, lr;                                                      // range of ranks, its size, index inside it
+      if (l < lfull) { t = l / (R * hpx); Rt = R; lr = l % (R * hpx); }
+      else { t = nfull; Rt = a.nqt - nfull * R; lr = l - lfull; }
+      const int gidx = lr / (Rt * Hg), rem = lr % (Rt * Hg);              // head group, index inside it (head-major)
+      rank = t * R + rem % Rt;
+      s = x + 8 * (gidx * Hg + rem / Rt);
     } else
 #endif
     { rank = blockIdx.x / U; s = blockIdx.x % U; }
