@@ -16,7 +16,7 @@ output type instead:
   * O = sum P8 * V8 and the denominator sum P8 (of the very same rounded values), fp32 accumulation on the GPU,
     float64 here; out = O / den * v_scale;  LSE2 = m + log2(sum of the unrounded p) - 5.
 
-Pinned in tests/test_oracle_attention.py: against brute-force Python loops on tiny shapes, and against
+Pinned in tests/test_oracle_fp8_model.py: against brute-force Python loops on tiny shapes, and against
 ``sage_reference`` on the fp8-dequantised V within the error that rounding P to 3 mantissa bits allows.
 """
 from __future__ import annotations
