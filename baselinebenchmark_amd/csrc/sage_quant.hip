@@ -205,8 +205,18 @@ __global__ void kmean_finalize_kernel(const double* partial, u16* km, int H, int
   if (cu_seqlens) L = cu_seqlens[b + 1] - cu_seqlens[b];
   if (d >= D) return;
   int nc = (L + kChunkRows - 1) / kChunkRows;
+  // eight partials in flight at a time (the loads are what this kernel waits for); still added in chunk order
+  const double* p = partial + (((int64_t)b * H + h) * nchunk) * D + d;
   double s = 0;
-  for (int c = 0; c < nc; c++) s += partial[(((int64_t)b * H + h) * nchunk + c) * D + d];
+  int c = 0;
+  for (; c + 8 <= nc; c += 8) {
+    double t[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) t[i] = p[(int64_t)(c + i) * D];
+#pragma unroll
+    for (int i = 0; i < 8; i++) s += t[i];
+  }
+  for (; c < nc; c++) s += p[(int64_t)c * D];
   float m = L > 0 ? (float)(s / (double)L) : 0.f;
   km[((int64_t)b * H + h) * D + d] = from_f32<DT>(m);
 }
@@ -218,8 +228,17 @@ __global__ void vscale_finalize_kernel(const float* partial, float* vscale, int 
   if (cu_seqlens) L = cu_seqlens[b + 1] - cu_seqlens[b];
   if (d >= D) return;
   int nc = (L + kChunkRows - 1) / kChunkRows;
+  const float* p = partial + (((int64_t)b * H + h) * nchunk) * D + d;
   float m = 0.f;
-  for (int c = 0; c < nc; c++) m = fmaxf(m, partial[(((int64_t)b * H + h) * nchunk + c) * D + d]);
+  int c = 0;
+  for (; c + 8 <= nc; c += 8) {
+    float t[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) t[i] = p[(int64_t)(c + i) * D];
+#pragma unroll
+    for (int i = 0; i < 8; i++) m = fmaxf(m, t[i]);
+  }
+  for (; c < nc; c++) m = fmaxf(m, p[(int64_t)c * D]);
   vscale[((int64_t)b * H + h) * D + d] = fmaxf(m / 448.0f, kScaleFloor);
 }
 
