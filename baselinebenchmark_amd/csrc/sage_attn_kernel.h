@@ -165,9 +165,10 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
   // coded without v_exp_f32 (FASTP, see softmax).
   constexpr bool RSUM = PV == 1;
   constexpr bool FASTP = PV == 1 && MSUM && MASK == 0;
-  // FP8 kernels take the row maximum in the vector phase (their softmax is short) and let the group that is in its
-  // vector phase issue the tile requests; FP16 kernels keep both in the matrix phase.
-  constexpr bool VECMAX = PV == 1;
+  // FP8 kernels, and FP16 ones of head_dim 128, take the row maximum in the vector phase and issue the tile requests at
+  // the end of group 0's matrix phase; FP16 kernels of head_dim 64 keep the row maximum in the matrix phase (their
+  // softmax, with its exponentials, is the longer one there: moving it measured -3 %, against +1 % at head_dim 128).
+  constexpr bool VECMAX = PV == 1 || D == 128;
 
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
@@ -796,7 +797,7 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
           SAGE_PH(3);
           even_barrier(j, issuer_in_flight(j));
           SAGE_PH(0);
-          if (j == 0) first_value_tile();   // V(0) has one period only: ahead of the first Q.K^T, not after it
+          if (LEAD == 2 && j == 0) first_value_tile();   // V(0) has one period only: ahead of the first Q.K^T, not after it
           if (j >= 1 && j - 1 < wnt) pv(j - 1);
           if (j < wnt) qk(j);
           request_tiles(j, false);
