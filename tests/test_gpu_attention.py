@@ -420,3 +420,35 @@ def test_config1_full_size_against_the_reference_formula():
         assert m["rel_rmse"] < 4e-3 and m["cosine"] >= 0.9999, (b, h, m)
         ms = oa.metrics(got, oa.sdpa_fp32(q1, k1, v1, "HND", True))
         assert ms["cosine"] >= 0.999, (b, h, ms)
+
+
+@pytest.mark.parametrize("pv,fused", [("fp16", False), ("fp8", False), ("fp8", True)])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("B,H,nqt", [(1, 8, 1), (1, 8, 3), (2, 8, 5), (1, 16, 16), (1, 8, 17), (1, 24, 33), (4, 32, 4)])
+def test_tile_order_inside_an_xcd_reaches_every_tile_exactly_once(pv, fused, causal, B, H, nqt):
+    """With a multiple of 8 heads the launch orders its q-tiles per XCD in tiers (consecutive q-tiles of a few heads at a
+    time); a single head per call takes the plain order.  Heads are independent, so the many-head call must equal, bit for
+    bit, the single-head calls on the same operands: every (head, q-tile) is computed exactly once and written where it
+    belongs.  Ragged last q-tile, 1 to 33 q-tiles per head, 8 to 128 heads; operands quantised once so that the
+    comparison is between launches of the attention kernel only."""
+    S, D = 256 * nqt - 56, 64
+    g = torch.Generator().manual_seed(77 + 13 * nqt + H)
+    q = randn("HND", B, H, S, D, torch.bfloat16, g).to(DEV)
+    k = randn("HND", B, H, S, D, torch.bfloat16, g).to(DEV)
+    v = randn("HND", B, H, S, D, torch.bfloat16, g).to(DEV)
+    qi, qs, ki, ks = sa.per_block_int8(q, k, BLKQ=64, BLKK=128)
+
+    def run(sl):
+        qq, kk, vv = (t[:, sl].contiguous() for t in (q, ki, v))
+        if fused:
+            o, _ = sa.forward_fused_q(qq, kk, vv, ks[:, sl].contiguous(), is_causal=causal, pv_mode=pv, BLKQ=64, BLKK=128)
+        else:
+            o, _ = sa.forward(qi[:, sl].contiguous(), kk, vv, qs[:, sl].contiguous(), ks[:, sl].contiguous(),
+                              output_dtype=torch.bfloat16, BLKQ=64, BLKK=128, is_causal=causal, pv_mode=pv)
+        return o
+
+    full = run(slice(0, H))
+    assert torch.isfinite(full.float()).all()
+    for h in sorted({0, 1, H // 2, H - 1}):
+        one = run(slice(h, h + 1))
+        assert torch.equal(full[:, h:h + 1], one), (h, (full[:, h:h + 1].float() - one.float()).abs().max().item())
