@@ -761,6 +761,11 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
     // V(j+LEAD-1), LEAD periods before their first use (a tile that has to come from HBM takes longer than one
     // period), into the slots whose last readers finished a barrier ago; with LEAD = 2, V(0) goes first in
     // period 0 and the requests of the last period may still be in flight at a barrier.
+    // FP16 kernels of head_dim 128 (twelve requests per period, the V tiles being twice as large) leave the V pieces of
+    // group 1's wavefronts to group 1, which requests them at the start of its matrix phase: both matrix phases then
+    // carry part of the requests instead of one carrying all of them (+2 % from 4k to 16k keys).
+    constexpr bool SPLIT_REQ = PV == 0 && VECMAX;
+    static_assert(!SPLIT_REQ || LEAD == 1, "group 1 requests V(j) in period j");
     auto first_value_tile = [&]() { load_v(0, 0); load_v(0, PARTNER); };
     auto request_tiles = [&](int j, bool with_first_value = true) {
 #ifdef SAGE_TIMING
@@ -769,7 +774,7 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
 #endif
       if (LEAD == 2 && j == 0 && with_first_value) first_value_tile();
       if (j + LEAD < ntiles) { load_k(j + LEAD, 0); load_k(j + LEAD, PARTNER); }
-      if (j + LEAD - 1 < ntiles) { load_v(j + LEAD - 1, 0); load_v(j + LEAD - 1, PARTNER); }
+      if (j + LEAD - 1 < ntiles) { load_v(j + LEAD - 1, 0); if (!SPLIT_REQ) load_v(j + LEAD - 1, PARTNER); }
 #ifdef SAGE_TIMING
       rq_sum += __builtin_amdgcn_s_memrealtime() - rq0;   // ticks this wavefront spent issuing the requests of a period
       rq_n++;
@@ -815,6 +820,7 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
           SAGE_PH(1);
           odd_barrier();
           SAGE_PH(2);
+          if (SPLIT_REQ && j < ntiles) load_v(j, PARTNER);   // V(j) of the pair's second wavefront: LEAD is 1 here
           if (j >= 1 && j - 1 < wnt) pv(j - 1);
           if (j < wnt) qk(j);
         }
