@@ -1,6 +1,7 @@
 """Where a q-tile's time goes inside the fused attention kernel: the timing build of the library stamps eight
 points of every workgroup on the GPU's constant-rate counter (entry, tile decoded, raw Q arrived, Q operand ready,
-first barrier of the main loop, main loop done, stores issued, stores acknowledged) and sums the intervals.
+first barrier of the main loop, main loop done, stores issued, stores acknowledged) and sums the intervals; the kernel's
+wall time says what a workgroup costs beyond them.
 
     python -m baselinebenchmark_amd.build --timing
     SAGE_MI355X_LIB=baselinebenchmark_amd/csrc/libsage_mi355x_timing.so python -m baselinebenchmark_amd.benchmarks.tile_timing
@@ -40,11 +41,22 @@ def measure(B, H, S, D, causal, dtype=torch.bfloat16, pv_mode="fp8", blkq=64, bl
     q, k, v = (torch.randn((B, H, S, D), dtype=dtype, device="cuda", generator=g) for _ in range(3))
     _, _, ki, ks = sa.per_block_int8(q, k, BLKQ=blkq, BLKK=blkk)
     call = lambda: sa.forward_fused_q(q, ki, v, ks, is_causal=causal, pv_mode=pv_mode, BLKQ=blkq, BLKK=blkk)
+    prep = lambda: sa.prepare_v(v, "HND", pv_mode)
     for _ in range(10):
         call()
+    # wall time of the attention kernel alone: the call minus its V preparation pass, HIP events on the current stream
+    def wall(fn):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(launches):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e6 / launches
+    prep()
+    t_prep = wall(prep)
     _read()
-    for _ in range(launches):
-        call()
+    t_call = wall(call)
     d = _read()
     rows = {}
     for cls, name in enumerate(("first wavefront", "last wavefront", "other wavefronts")):
@@ -58,6 +70,12 @@ def measure(B, H, S, D, causal, dtype=torch.bfloat16, pv_mode="fp8", blkq=64, bl
         rows[f"group {g} phases"] = [d[32 + 4 * g + k] * TICK_NS / n for k in range(4)]
     rows["request issue"] = [d[42] * TICK_NS / max(d[43], 1)]
     rows["raw Q wait"] = [d[44] * TICK_NS / max(d[45], 1)]
+    # what a workgroup's slot on a compute unit costs beyond the time its wavefronts measure themselves: the kernel's
+    # wall time divided by the workgroups a compute unit runs one after the other, minus a workgroup's own total
+    cus = torch.cuda.get_device_properties(q.device).multi_processor_count
+    per_cu = B * H * ((S + 255) // 256) / cus
+    own = sum(rows["other wavefronts"])
+    rows["between workgroups"] = [t_call - t_prep, per_cu, (t_call - t_prep) / per_cu - own]
     return rows, tiles
 
 
@@ -77,6 +95,10 @@ def main():
                 continue
             if len(vals) == 1:
                 print(f"  {name:17s} {vals[0]:.0f} ns per period for the wavefront that issues the tile requests", flush=True)
+                continue
+            if name == "between workgroups":
+                print(f"  {name:17s} kernel {vals[0] / 1e3:.0f} us for {vals[1]:.1f} workgroups per compute unit: "
+                      f"{vals[2]:.0f} ns per workgroup beyond its own stamps (dispatch, wavefront start-up, imbalance)", flush=True)
                 continue
             if len(vals) == 4:
                 print(f"  {name:17s} per period {sum(vals):6.0f} ns | first phase {vals[0]:.0f}, odd barrier {vals[1]:.0f}, "

@@ -133,7 +133,11 @@ constexpr int attn_lds_bytes() { return attn_tile_lds_bytes<D, NW, BN, PV, CAUSA
 // [42] / [43] = ticks per period that the issuing wavefront spends on the tile requests; [44] / [45] = ticks a wavefront
 // of the kernels that quantise their own Q waits, after its last prologue request, for the raw rows to arrive.
 #ifdef SAGE_TIMING
-static __device__ unsigned long long g_tile_timing[48];
+// The sums are kept in kTimingSets copies, one per workgroup index modulo kTimingSets, and added up on the host: with a
+// single copy the atomics of thousands of short workgroups pile up on three cache lines and hold up the L2 channel
+// they live in, tile requests included.
+constexpr int kTimingSets = 256;
+static __device__ unsigned long long g_tile_timing[kTimingSets][48];
 #define SAGE_PH(k) do { const long long t_ = __builtin_amdgcn_s_memrealtime(); if (ph_last) ph_sum[((k) + 3) & 3] += t_ - ph_last; ph_last = t_; if ((k) == 0) ph_n++; } while (0)
 #define SAGE_T(k, x) do { asm volatile("" : "+v"(x)); sage_ts[k] = __builtin_amdgcn_s_memrealtime(); } while (0)
 #else
@@ -201,7 +205,7 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
       // finish together.  Long sequences get R = 32: one head at a time.  The q-tiles of a head walk the same K/V
       // tiles from tile 0 on at about the same pace, so one of them fetches a tile into the XCD's L2 and the others
       // hit it there (a quarter of the L2 fills of the plain heaviest-first order, where an XCD works on all its heads
-      // at once), and neighbouring q-tiles read neighbouring rows of Q (the raw Q tile arrives in about half the time).
+      // at once), and neighbouring q-tiles read neighbouring rows of Q.
       const int x = blockIdx.x & 7, l = blockIdx.x >> 3, hpx = U >> 3;   // XCD, index inside it, heads per XCD
       int R = 32;
       while (R > 1 && 2 * R > a.nqt) R >>= 1;
@@ -945,18 +949,19 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
   sage_ts[7] = __builtin_amdgcn_s_memrealtime();   // stores acknowledged
   if (ntiles == 0) sage_ts[4] = sage_ts[3];
   if (lane == 0) {
+    unsigned long long* tt = g_tile_timing[blockIdx.x % kTimingSets];
     const int cls = w == 0 ? 0 : (w == NW - 1 ? 1 : 2);
-    for (int i = 0; i < 7; i++) atomicAdd(&g_tile_timing[cls * 8 + i], (unsigned long long)(sage_ts[i + 1] - sage_ts[i]));
-    atomicAdd(&g_tile_timing[cls * 8 + 7], 1ull);
-    if (w == 0) atomicAdd(&g_tile_timing[24], (unsigned long long)ntiles);
+    for (int i = 0; i < 7; i++) atomicAdd(&tt[cls * 8 + i], (unsigned long long)(sage_ts[i + 1] - sage_ts[i]));
+    atomicAdd(&tt[cls * 8 + 7], 1ull);
+    if (w == 0) atomicAdd(&tt[24], (unsigned long long)ntiles);
     if (w == 1 || w == NW - 2) {   // one wavefront of each group
       const int g = (w >> GSH) & 1;
-      for (int i = 0; i < 4; i++) atomicAdd(&g_tile_timing[32 + 4 * g + i], (unsigned long long)ph_sum[i]);
-      atomicAdd(&g_tile_timing[40 + g], (unsigned long long)ph_n);
-      atomicAdd(&g_tile_timing[42], (unsigned long long)rq_sum);   // [42] / [43]: ticks per period spent issuing the tile requests
-      atomicAdd(&g_tile_timing[43], (unsigned long long)rq_n);
-      atomicAdd(&g_tile_timing[44], (unsigned long long)q_wait);   // [44] / [45]: ticks a wavefront waits for its raw Q rows (and the first K tile)
-      atomicAdd(&g_tile_timing[45], 1ull);
+      for (int i = 0; i < 4; i++) atomicAdd(&tt[32 + 4 * g + i], (unsigned long long)ph_sum[i]);
+      atomicAdd(&tt[40 + g], (unsigned long long)ph_n);
+      atomicAdd(&tt[42], (unsigned long long)rq_sum);   // [42] / [43]: ticks per period spent issuing the tile requests
+      atomicAdd(&tt[43], (unsigned long long)rq_n);
+      atomicAdd(&tt[44], (unsigned long long)q_wait);   // [44] / [45]: ticks a wavefront waits for its raw Q rows (and the first K tile)
+      atomicAdd(&tt[45], 1ull);
     }
   }
 #endif

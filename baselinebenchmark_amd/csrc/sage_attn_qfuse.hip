@@ -1,6 +1,7 @@
 // Fused attention kernel variants that quantise their own Q tile in the prologue (the one-call
 // pipeline skips the separate pass over Q: one HBM round trip less).  Own translation unit so that
 // the sets of instantiations compile in parallel.
+#include <cstring>
 #include "sage_attn_kernel.h"
 
 namespace sage {
@@ -19,9 +20,14 @@ hipError_t launch_attn_qfused(const AttnArgs& a, int D, int pv, bool causal, int
 // Timing build only: copies the interval sums of the kernels of this translation unit (the ones the one-call
 // pipeline runs) to `out` (48 values) and clears them.  Synchronises the device.
 extern "C" int sage_tile_timing(unsigned long long* out) {
-  static const unsigned long long zero[48] = {};
+  static unsigned long long sets[sage::kTimingSets][48];
   if (hipDeviceSynchronize() != hipSuccess) return -1;
-  if (hipMemcpyFromSymbol(out, HIP_SYMBOL(sage::g_tile_timing), sizeof(zero)) != hipSuccess) return -1;
-  return hipMemcpyToSymbol(HIP_SYMBOL(sage::g_tile_timing), zero, sizeof(zero)) == hipSuccess ? 0 : -1;
+  if (hipMemcpyFromSymbol(sets, HIP_SYMBOL(sage::g_tile_timing), sizeof(sets)) != hipSuccess) return -1;
+  for (int i = 0; i < 48; i++) {
+    out[i] = 0;
+    for (int s = 0; s < sage::kTimingSets; s++) out[i] += sets[s][i];
+  }
+  memset(sets, 0, sizeof(sets));
+  return hipMemcpyToSymbol(HIP_SYMBOL(sage::g_tile_timing), sets, sizeof(sets)) == hipSuccess ? 0 : -1;
 }
 #endif
