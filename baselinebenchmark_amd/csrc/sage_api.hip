@@ -34,6 +34,9 @@ bool valid_blk_quant(int blk) { return blk == 16 || blk == 32 || blk == 64 || bl
 bool valid_blk_attn(int blk) { return blk == 16 || blk == 32 || blk == 64 || blk == 128; }
 bool valid_blkk_attn(int blk) { return valid_blk_attn(blk); }
 int ilog2(int x) { int r = 0; while ((1 << r) < x) r++; return r; }
+// A Q block-size argument may carry SAGE_BLK_INTERLEAVE8: eight interleaved scales per block instead of one.
+int blk_rows(int blk) { return blk > 0 ? (blk & ~SAGE_BLK_INTERLEAVE8) : blk; }
+int blk_groups(int blk) { return (blk > 0 && (blk & SAGE_BLK_INTERLEAVE8)) ? 8 : 1; }
 
 int check_common(int B, int H, int L, int D, int dtype) {
   if (B < 0 || H < 0 || L < 0) return fail(SAGE_EINVAL, "negative dimension (B=%d H=%d L=%d)", B, H, L);
@@ -76,7 +79,11 @@ int quant_impl(const void* x, int8_t* out, float* scale, const void* km, int B, 
                float mult, int dtype, const int32_t* cu_seqlens, const int32_t* cu_blocks, int64_t scale_sh,
                const RowDot& dot, sage_stream_t stream) {
   if (int rc = check_common(B, H, L, D, dtype)) return rc;
+  const int groups = blk_groups(blk);
+  blk = blk_rows(blk);
   if (!valid_blk_quant(blk)) return fail(SAGE_ENOTIMPL, "quantisation block %d is not supported (16, 32, 64, 128)", blk);
+  if (groups > 1 && cu_seqlens) return fail(SAGE_ENOTIMPL, "interleaved scales are not supported for packed batches");
+  if (groups > 1 && km) return fail(SAGE_ENOTIMPL, "interleaved scales are a Q granularity: not together with a K mean");
   if (B == 0 || H == 0 || L == 0) return SAGE_OK;
   if (!x || !out || !scale) return fail(SAGE_EINVAL, "null tensor pointer");
   if (cu_seqlens && !cu_blocks) return fail(SAGE_EINVAL, "packed mode needs cu_blocks");
@@ -88,7 +95,7 @@ int quant_impl(const void* x, int8_t* out, float* scale, const void* km, int B, 
   a.x = (const u16*)x; a.out = out; a.scale = scale; a.km = (const u16*)km;
   a.B = B; a.H = H; a.L = L; a.D = D;
   a.x_sb = x_sb; a.x_sh = x_sh; a.x_sn = x_sn; a.o_sb = o_sb; a.o_sh = o_sh; a.o_sn = o_sn;
-  a.km_sb = km_sb; a.km_sh = km_sh; a.blk = blk; a.mult = mult;
+  a.km_sb = km_sb; a.km_sh = km_sh; a.blk = blk; a.groups = groups; a.mult = mult;
   a.cu_seqlens = cu_seqlens; a.cu_blocks = cu_blocks; a.scale_sh = scale_sh;
   a.dotv = (const u16*)dot.vec; a.dot_out = dot.out; a.dv_sb = dot.sb; a.dv_sh = dot.sh; a.dv_group = dot.group;
   a.dot_total = dot.total;
@@ -213,8 +220,12 @@ int attn_impl(const int8_t* q, const int8_t* k, const void* v_panels, const floa
   if (Hkv <= 0 || Hq % Hkv) return fail(SAGE_EINVAL, "query heads (%d) must be divisible by KV heads (%d)", Hq, Hkv);
   if (Skv < 0) return fail(SAGE_EINVAL, "negative kv length");
   if (pv_mode != SAGE_PV_FP16 && pv_mode != SAGE_PV_FP8) return fail(SAGE_EINVAL, "pv_mode %d unknown", pv_mode);
+  const int qgroups = blk_groups(blkq);
+  blkq = blk_rows(blkq);
   if (!valid_blk_attn(blkq) || !valid_blkk_attn(blkk))
     return fail(SAGE_ENOTIMPL, "attention needs Q and K scale blocks of 16, 32, 64 or 128 rows (got %d/%d)", blkq, blkk);
+  if (qgroups > 1 && cu_seqlens_q) return fail(SAGE_ENOTIMPL, "interleaved Q scales are not supported for packed batches");
+  if (qgroups > 1 && qraw.ptr) return fail(SAGE_ENOTIMPL, "interleaved Q scales need the standalone Q quantiser (sage_quant_int8)");
   if (blkk == 16 && mask.ptr) return fail(SAGE_ENOTIMPL, "K scale blocks of 16 rows cannot be combined with an explicit mask");
   if (B == 0 || Hq == 0 || Sq == 0) return SAGE_OK;
   if (!out || (Skv > 0 && (!k || !v_panels || !k_scale))) return fail(SAGE_EINVAL, "null tensor pointer");
@@ -245,7 +256,8 @@ int attn_impl(const int8_t* q, const int8_t* k, const void* v_panels, const floa
   a.B = B; a.Hq = Hq; a.Hkv = Hkv; a.Sq = Sq; a.Skv = Skv;
   a.q_sb = q_sb; a.q_sh = q_sh; a.q_sn = q_sn; a.k_sb = k_sb; a.k_sh = k_sh; a.k_sn = k_sn;
   a.o_sb = o_sb; a.o_sh = o_sh; a.o_sn = o_sn;
-  a.blkq = blkq; a.blkk = blkk; a.blkq_shift = ilog2(blkq); a.blkk_shift = ilog2(blkk); a.out_bf16 = out_dtype == SAGE_DT_BF16;
+  a.blkq = blkq; a.blkk = blkk; a.blkq_shift = ilog2(blkq); a.blkk_shift = ilog2(blkk); a.qg_shift = qgroups == 8 ? 3 : 0;
+  a.out_bf16 = out_dtype == SAGE_DT_BF16;
   a.nqt = (Sq + BM - 1) / BM;
   a.mask = mask.ptr; a.mask_kind = mask.kind; a.m_sb = mask.sb; a.m_sh = mask.sh; a.m_sm = mask.sm; a.m_sn = mask.sn;
   a.mask_mult = mask.mult; a.lse_offset = lse_offset;
@@ -322,12 +334,12 @@ E2EWorkspace e2e_layout(int B, int Hq, int Hkv, int Sq, int Skv, int D, int blkq
   w.q_i8 = off; off += align_up(nq);
   w.k_i8 = off; off += align_up(nk);
   if (varlen) {
-    w.qs_sh = total_q / blkq + B; w.ks_sh = total_k / blkk + B; w.panel_sh = total_k / SAGE_PANEL_ROWS + B;
+    w.qs_sh = total_q / blk_rows(blkq) + B; w.ks_sh = total_k / blkk + B; w.panel_sh = total_k / SAGE_PANEL_ROWS + B;
     w.q_scale = off; off += align_up((size_t)Hq * w.qs_sh * 4);
     w.k_scale = off; off += align_up((size_t)Hkv * w.ks_sh * 4);
   } else {
     w.qs_sh = w.ks_sh = w.panel_sh = 0;
-    w.q_scale = off; off += align_up((size_t)B * Hq * ((Sq + blkq - 1) / blkq) * 4);
+    w.q_scale = off; off += align_up((size_t)B * Hq * ((Sq + blk_rows(blkq) - 1) / blk_rows(blkq)) * blk_groups(blkq) * 4);
     w.k_scale = off; off += align_up((size_t)B * Hkv * ((Skv + blkk - 1) / blkk) * 4);
   }
   w.km = off; off += align_up((size_t)B * Hkv * D * 2);
@@ -369,10 +381,11 @@ int sage_sageattn_masked(const void* q, const void* k, const void* v, void* out,
                          int64_t m_sm, int64_t m_sn, sage_stream_t stream) {
   if (int rc = check_common(B, Hq, Sq, D, dtype)) return rc;
   if (Hkv <= 0 || Hq % Hkv) return fail(SAGE_EINVAL, "query heads (%d) must be divisible by KV heads (%d)", Hq, Hkv);
-  if (!valid_blk_attn(blkq) || !valid_blkk_attn(blkk))
-    return fail(SAGE_ENOTIMPL, "Q and K scale blocks must be 16, 32, 64 or 128 rows (got %d/%d)", blkq, blkk);
+  if (!valid_blk_attn(blk_rows(blkq)) || !valid_blkk_attn(blkk))
+    return fail(SAGE_ENOTIMPL, "Q and K scale blocks must be 16, 32, 64 or 128 rows (got %d/%d)", blk_rows(blkq), blkk);
   if (pv_mode != SAGE_PV_FP16 && pv_mode != SAGE_PV_FP8) return fail(SAGE_EINVAL, "pv_mode %d unknown", pv_mode);
   const int varlen = cu_seqlens_q != nullptr;
+  if (varlen && blk_groups(blkq) > 1) return fail(SAGE_ENOTIMPL, "interleaved Q scales are not supported for packed batches");
   if (varlen && !cu_seqlens_k) return fail(SAGE_EINVAL, "packed mode needs cu_seqlens_k");
   if (B == 0 || Hq == 0 || Sq == 0) return SAGE_OK;
   if (!workspace) return fail(SAGE_EWORKSPACE, "null workspace");
@@ -427,7 +440,7 @@ int sage_sageattn_masked(const void* q, const void* k, const void* v, void* out,
   // Q is quantised by the attention kernel itself (each q-tile exactly where it is consumed) unless a
   // feature needs the standalone pass: an explicit mask or the LSE correction.
   const float q_mult = (float)((sm_scale > 0 ? sm_scale : 1.0 / sqrt((double)D)) * 1.44269504);
-  const bool fuse_q = !attn_mask && !lse_off;
+  const bool fuse_q = !attn_mask && !lse_off && blk_groups(blkq) == 1;   // (interleaved scales: standalone pass too)
   if (!fuse_q) {
     rc = quant_impl(q, q_i8, q_scale, nullptr, B, Hq, Sq, D, q_sb, q_sh, q_sn, qi_sb, qi_sh, qi_sn, 0, 0, blkq, q_mult, dtype,
                     cu_seqlens_q, cu_qblk, w.qs_sh, dot, stream);

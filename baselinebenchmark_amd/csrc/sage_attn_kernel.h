@@ -254,7 +254,7 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
     ooff = (int64_t)b * a.o_sb + (int64_t)hq * a.o_sh;
     koff = (int64_t)b * a.k_sb + (int64_t)kvh * a.k_sh;
     lseoff = ((int64_t)b * a.Hq + hq) * a.Sq;
-    qsp = a.qs + ((int64_t)b * a.Hq + hq) * ((Lq + a.blkq - 1) / a.blkq);
+    qsp = a.qs + (((int64_t)b * a.Hq + hq) * ((Lq + a.blkq - 1) / a.blkq) << a.qg_shift);
     ksp = a.ks + ((int64_t)b * a.Hkv + kvh) * ((Lk + a.blkk - 1) / a.blkk);
     vbase = a.vp + ((int64_t)b * a.Hkv + kvh) * ((Lk + kPanelRows - 1) / kPanelRows) * PANEL_BYTES;
   }
@@ -346,7 +346,10 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
     const int8_t* qp = a.q + qoff + (int64_t)min(my_row, Lq - 1) * a.q_sn + 16 * h;
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) qreg[ks] = *reinterpret_cast<const v4i*>(qp + 32 * ks);
-    qscale = qsp[min(my_row, Lq - 1) >> a.blkq_shift];   // per lane: scale blocks may be smaller than a wavefront's 32 rows
+    // per lane: scale blocks may be smaller than a wavefront's 32 rows, and with interleaved scales the rows r, r + 8, ...
+    // of a block share one of its eight
+    const int qrow = min(my_row, Lq - 1);
+    qscale = qsp[((qrow >> a.blkq_shift) << a.qg_shift) + (qrow & ((1 << a.qg_shift) - 1))];
   } else {
     // Quantise this wavefront's 32 rows here, exactly as quant_int8_kernel would
     // (quant_per_block.py:38-46): x32 = fp32(x) * mult, scale = max|x32| / 127 over the scale block

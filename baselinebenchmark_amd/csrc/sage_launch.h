@@ -12,6 +12,7 @@ struct QuantArgs {
   int B, H, L, D;
   int64_t x_sb, x_sh, x_sn, o_sb, o_sh, o_sn, km_sb, km_sh;
   int blk;
+  int groups;   // scales per block: 1, or 8 (scale g covers the rows r of the block with r % 8 == g); fixed-length only
   float mult;
   const int32_t* cu_seqlens;
   const int32_t* cu_blocks;
@@ -58,6 +59,7 @@ struct AttnArgs {
   int64_t q_sb, q_sh, q_sn, k_sb, k_sh, k_sn, o_sb, o_sh, o_sn;
   int blkq, blkk;            // scale block sizes: powers of two (32, 64, 128)
   int blkq_shift, blkk_shift;  // their log2
+  int qg_shift;              // log2 of the Q scales per block: 0, or 3 (eight interleaved scales: rows r, r + 8, ... share one)
   int out_bf16;
   int nqt;  // q-tiles per sequence (fixed-length mode)
   // packed mode (cu_q != nullptr)

@@ -38,7 +38,7 @@ __global__ void __launch_bounds__(256) quant_int8_kernel(QuantArgs a) {
   } else {
     xbase = (int64_t)b * a.x_sb + (int64_t)h * a.x_sh;
     obase = (int64_t)b * a.o_sb + (int64_t)h * a.o_sh;
-    sidx = ((int64_t)b * a.H + h) * ((L + a.blk - 1) / a.blk) + blkid;
+    sidx = (((int64_t)b * a.H + h) * ((L + a.blk - 1) / a.blk) + blkid) * a.groups;
     dbase = ((int64_t)b * a.H + h) * L;
   }
   const int n0 = blkid * a.blk;
@@ -105,12 +105,28 @@ __global__ void __launch_bounds__(256) quant_int8_kernel(QuantArgs a) {
     }
   }
   __shared__ float wmax[4];
-  amax = wave_max(amax);
-  if ((tid & 63) == 0) wmax[tid >> 6] = amax;
-  __syncthreads();
-  amax = fmaxf(fmaxf(wmax[0], wmax[1]), fmaxf(wmax[2], wmax[3]));
+  __shared__ int gmax[8];
+  if (a.groups == 1) {
+    amax = wave_max(amax);
+    if ((tid & 63) == 0) wmax[tid >> 6] = amax;
+    __syncthreads();
+    amax = fmaxf(fmaxf(wmax[0], wmax[1]), fmaxf(wmax[2], wmax[3]));
+  } else {
+    // Eight interleaved scales per block: every row this lane holds has the same index modulo 8 (the passes are
+    // RPP rows apart, a multiple of 8), so the lane belongs to one group.  Maximum over the lanes of a row, then over
+    // the rows of the group through LDS (the values are non-negative floats: their bit patterns order like integers).
+    static_assert(RPP % 8 == 0, "a lane's rows must share their index modulo 8");
+    if (tid < 8) gmax[tid] = 0;
+    __syncthreads();
+#pragma unroll
+    for (int o = 1; o < TPR; o <<= 1) amax = fmaxf(amax, __shfl_xor(amax, o));
+    if (tc == 0) atomicMax(&gmax[tr & 7], __builtin_bit_cast(int, amax));
+    __syncthreads();
+    amax = __builtin_bit_cast(float, gmax[tr & 7]);
+  }
   const float scale = fmaxf(amax / 127.0f, kScaleFloor);
-  if (tid == 0) a.scale[sidx] = scale;
+  if (a.groups == 1) { if (tid == 0) a.scale[sidx] = scale; }
+  else if (tc == 0 && tr < 8) a.scale[sidx + tr] = scale;
 
   const float rcp = 1.0f / scale;
   // The fast correction-step division needs: significand of scale not all ones, and scale and rcp

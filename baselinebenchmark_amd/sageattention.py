@@ -98,11 +98,20 @@ def k_mean(k: torch.Tensor, tensor_layout: str = "HND") -> torch.Tensor:
     return km.view(B, H, 1, D) if tensor_layout == "HND" else km.view(B, 1, H, D)
 
 
-def _quant_one(x, km, blk, mult, tensor_layout):
+BLK_INTERLEAVE8 = 0x100   # SAGE_BLK_INTERLEAVE8 of the C ABI: eight interleaved scales per Q block
+
+
+def _check_interleave(q_interleave) -> int:
+    if q_interleave not in (1, 8):
+        raise ValueError("q_interleave must be 1 (one scale per Q block) or 8 (rows r, r+8, ... of a block share a scale)")
+    return BLK_INTERLEAVE8 if q_interleave == 8 else 0
+
+
+def _quant_one(x, km, blk, mult, tensor_layout, groups=1):
     B, H, L, D, sb, sh, sn = _layout(x, tensor_layout)
     out = torch.empty(x.shape, device=x.device, dtype=torch.int8)
     _, _, _, _, osb, osh, osn = _layout(out, tensor_layout)
-    scale = torch.empty((B, H, (L + blk - 1) // blk), device=x.device, dtype=torch.float32)
+    scale = torch.empty((B, H, (L + blk - 1) // blk * groups), device=x.device, dtype=torch.float32)
     km_sb = km_sh = 0
     if km is not None:
         if km.dtype != x.dtype or km.device != x.device:
@@ -112,16 +121,19 @@ def _quant_one(x, km, blk, mult, tensor_layout):
             km = km.contiguous()
         km_sb, km_sh = (km.stride(0), km.stride(1)) if tensor_layout == "HND" else (km.stride(0), km.stride(2))
     check(lib().sage_quant_int8(_ptr(x), _ptr(out), _ptr(scale), _ptr(km), B, H, L, D, sb, sh, sn, osb, osh, osn,
-                                km_sb, km_sh, blk, mult, _dt(x.dtype), None, None, 0, _stream(x)))
+                                km_sb, km_sh, blk | _check_interleave(groups), mult, _dt(x.dtype), None, None, 0, _stream(x)))
     return out, scale
 
 
 @torch.no_grad()
-def per_block_int8(q, k, km=None, BLKQ=128, BLKK=64, sm_scale=None, tensor_layout="HND"):
+def per_block_int8(q, k, km=None, BLKQ=128, BLKK=64, sm_scale=None, tensor_layout="HND", q_interleave=1):
     """Per-block INT8 quantisation of Q and K; returns (q_int8, q_scale, k_int8, k_scale).
 
     Same contract as quant_per_block.py:49-101: optional ``k - km`` in the input dtype, Q scaled by
     ``sm_scale * 1.44269504`` (default sm_scale = head_dim**-0.5), K by 1, scales [B, H, ceil(L/BLK)].
+    ``q_interleave=8`` (no counterpart in the reference's code; the granularity upstream SageAttention calls per-thread,
+    with WARPQ = BLKQ): every Q block gets eight scales, scale g for its rows r with r % 8 == g, and q_scale is
+    [B, H, ceil(L/BLKQ) * 8]; pass the same keyword to ``forward``.
     """
     _check_float("q", q)
     _check_float("k", k)
@@ -134,7 +146,8 @@ def per_block_int8(q, k, km=None, BLKQ=128, BLKK=64, sm_scale=None, tensor_layou
     if q.shape[-1] != k.shape[-1]:
         raise ValueError("q and k head dimensions differ")
     _check_blocks_quant(BLKQ, BLKK)
-    q_int8, q_scale = _quant_one(q, None, BLKQ, _q_mult(q.shape[-1], sm_scale), tensor_layout)
+    _check_interleave(q_interleave)
+    q_int8, q_scale = _quant_one(q, None, BLKQ, _q_mult(q.shape[-1], sm_scale), tensor_layout, q_interleave)
     k_int8, k_scale = _quant_one(k, km, BLKK, 1.0, tensor_layout)
     return q_int8, q_scale, k_int8, k_scale
 
@@ -199,7 +212,7 @@ def _mask_args(attn_mask, B, Hq, Sq, Skv, device):
 @torch.no_grad()
 def forward(q, k, v, q_scale, k_scale, tensor_layout="HND", attn_mask=None, output_dtype=torch.float16,
             return_lse=False, maxnreg=None, block_m=None, num_warps=None, num_stages=None, backend=None,
-            BLKQ=128, BLKK=64, is_causal=False, pv_mode="fp16"):
+            BLKQ=128, BLKK=64, is_causal=False, pv_mode="fp16", q_interleave=1):
     """Fused INT8-QK attention on operands produced by per_block_int8; returns (out, lse).
 
     Signature of sageattention_hip.py:55-56 / attn_qk_int8_per_block_native.py:438-453; the tuning
@@ -209,7 +222,9 @@ def forward(q, k, v, q_scale, k_scale, tensor_layout="HND", attn_mask=None, outp
     ``attn_mask``: boolean (True keeps the key) or additive bias on the base-2 logits, broadcastable
     to [B, Hq, Sq, Skv] (sageattention_triton.py:92-105); not combinable with ``is_causal``.
     ``lse`` is base 2 (sageattention_triton.py:127-129) and an empty tensor unless requested.
+    ``q_interleave=8``: q_scale holds eight interleaved scales per Q block (see per_block_int8).
     """
+    qflag = _check_interleave(q_interleave)
     for name, t in (("q", q), ("k", k)):
         if not isinstance(t, torch.Tensor) or not t.is_cuda or t.dtype != torch.int8 or not t.is_contiguous():
             raise TypeError(f"{name} must be contiguous GPU INT8")
@@ -235,7 +250,7 @@ def forward(q, k, v, q_scale, k_scale, tensor_layout="HND", attn_mask=None, outp
         raise NotImplementedError("head_dim must be 64 or 128")
     if BLKQ not in (16, 32, 64, 128) or BLKK not in (16, 32, 64, 128):
         raise NotImplementedError("the attention kernel needs Q and K scale blocks of 16, 32, 64 or 128 rows")
-    exp_q = (B, Hq, (Sq + BLKQ - 1) // BLKQ)
+    exp_q = (B, Hq, (Sq + BLKQ - 1) // BLKQ * q_interleave)
     exp_k = (B, Hkv, (Skv + BLKK - 1) // BLKK)
     if tuple(q_scale.shape) != exp_q:
         raise ValueError(f"q_scale has shape {tuple(q_scale.shape)}, expected {exp_q}")
@@ -255,13 +270,13 @@ def forward(q, k, v, q_scale, k_scale, tensor_layout="HND", attn_mask=None, outp
                                          _ptr(k_scale.contiguous()), _ptr(v_scale), _ptr(out),
                                          _ptr(lse if return_lse else None),
                                          B, Hq, Hkv, Sq, Skv, D, qsb, qsh, qsn, ksb, ksh, ksn, osb, osh, osn,
-                                         BLKQ, BLKK, pv, _dt(output_dtype), _ptr(m), kind, ms[0], ms[1], ms[2], ms[3],
+                                         BLKQ | qflag, BLKK, pv, _dt(output_dtype), _ptr(m), kind, ms[0], ms[1], ms[2], ms[3],
                                          _stream(q)))
         return out, lse
     check(lib().sage_attn_fwd(_ptr(q), _ptr(k), _ptr(panels), _ptr(q_scale.contiguous()), _ptr(k_scale.contiguous()),
                               _ptr(v_scale), _ptr(out), _ptr(lse if return_lse else None),
                               B, Hq, Hkv, Sq, Skv, D, qsb, qsh, qsn, ksb, ksh, ksn, osb, osh, osn,
-                              BLKQ, BLKK, int(bool(is_causal)), pv, _dt(output_dtype),
+                              BLKQ | qflag, BLKK, int(bool(is_causal)), pv, _dt(output_dtype),
                               None, None, None, 0, 0, 0, 0, _stream(q)))
     return out, lse
 
@@ -331,7 +346,7 @@ def _apply_recipe(quant_recipe, BLKQ, BLKK, pv_mode):
 @torch.no_grad()
 def sageattn(q, k, v, tensor_layout="HND", is_causal=False, sm_scale=None, smooth_k=True, pv_mode=None,
              BLKQ=128, BLKK=64, return_lse=False, qk_quant_dtype="int8", quant_recipe=None, attn_mask=None,
-             cu_seqlens_q=None, cu_seqlens_k=None, max_seqlen_q=None, max_seqlen_k=None, **kwargs):
+             cu_seqlens_q=None, cu_seqlens_k=None, max_seqlen_q=None, max_seqlen_k=None, q_interleave=1, **kwargs):
     """Quantise + attend in one call: out = softmax(q k^T * sm_scale [causal | + attn_mask]) v.
 
     Returns ``out`` (q's shape and dtype), or ``(out, lse)`` with ``return_lse=True`` where lse is
@@ -346,13 +361,17 @@ def sageattn(q, k, v, tensor_layout="HND", is_causal=False, sm_scale=None, smoot
     q is then [total_q, Hq, D], k and v [total_k, Hkv, D], ``tensor_layout`` is not consulted, ``max_seqlen_q`` /
     ``max_seqlen_k`` bound the sequence lengths (derived from cu_seqlens, with one host synchronisation, when left
     out), and lse comes back as [Hq, total_q]; see sageattn_varlen, which this call is then identical to.
+    ``q_interleave=8``: eight interleaved Q scales per block (see per_block_int8); fixed-length batches only.
     """
     if qk_quant_dtype != "int8":
         raise NotImplementedError("only INT8 Q/K quantisation is implemented")
     if kwargs:
         raise TypeError(f"unexpected arguments: {sorted(kwargs)}")
     BLKQ, BLKK, pv_mode = _apply_recipe(quant_recipe, BLKQ, BLKK, pv_mode)
+    qflag = _check_interleave(q_interleave)
     if cu_seqlens_q is not None or cu_seqlens_k is not None:
+        if qflag:
+            raise NotImplementedError("interleaved Q scales are not supported for packed batches")
         if attn_mask is not None:
             raise NotImplementedError("attn_mask is not supported for packed batches")
         cu_seqlens_k = cu_seqlens_q if cu_seqlens_k is None else cu_seqlens_k
@@ -387,7 +406,7 @@ def sageattn(q, k, v, tensor_layout="HND", is_causal=False, sm_scale=None, smoot
     out = torch.empty(q.shape, device=q.device, dtype=q.dtype)
     _, _, _, _, osb, osh, osn = _layout(out, tensor_layout)
     lse = torch.empty((B, Hq, Sq), device=q.device, dtype=torch.float32) if return_lse else None
-    ws_bytes = lib().sage_sageattn_workspace_bytes(B, Hq, Hkv, Sq, Skv, D, BLKQ, BLKK, pv, 0, 0, 0)
+    ws_bytes = lib().sage_sageattn_workspace_bytes(B, Hq, Hkv, Sq, Skv, D, BLKQ | qflag, BLKK, pv, 0, 0, 0)
     ws = torch.empty(max(ws_bytes, 256), device=q.device, dtype=torch.uint8)
     if attn_mask is not None:
         if is_causal:
@@ -395,13 +414,13 @@ def sageattn(q, k, v, tensor_layout="HND", is_causal=False, sm_scale=None, smoot
         m, kind, ms = _mask_args(attn_mask, B, Hq, Sq, Skv, q.device)
         check(lib().sage_sageattn_masked(_ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _ptr(ws), ws_bytes,
                                          B, Hq, Hkv, Sq, Skv, D, qsb, qsh, qsn, ksb, ksh, ksn, vsb, vsh, vsn, osb, osh, osn,
-                                         _dt(q.dtype), BLKQ, BLKK, float(D ** -0.5 if sm_scale is None else sm_scale),
+                                         _dt(q.dtype), BLKQ | qflag, BLKK, float(D ** -0.5 if sm_scale is None else sm_scale),
                                          0, int(bool(smooth_k)), pv, None, None, 0, 0,
                                          _ptr(m), kind, ms[0], ms[1], ms[2], ms[3], _stream(q)))
     else:
         check(lib().sage_sageattn(_ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _ptr(ws), ws_bytes,
                                   B, Hq, Hkv, Sq, Skv, D, qsb, qsh, qsn, ksb, ksh, ksn, vsb, vsh, vsn, osb, osh, osn,
-                                  _dt(q.dtype), BLKQ, BLKK, float(D ** -0.5 if sm_scale is None else sm_scale),
+                                  _dt(q.dtype), BLKQ | qflag, BLKK, float(D ** -0.5 if sm_scale is None else sm_scale),
                                   int(bool(is_causal)), int(bool(smooth_k)), pv, None, None, 0, 0, _stream(q)))
     if return_lse:
         return out, lse * 0.6931471805599453

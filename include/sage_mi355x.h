@@ -42,6 +42,18 @@ extern "C" {
 #define SAGE_MASK_BOOL 1     /* bytes; non-zero = the key is visible (torch.bool)                */
 #define SAGE_MASK_ADDITIVE 2 /* fp32 bias added to the logits                                    */
 
+/* Interleaved ("per-thread") Q scales.  OR-ed into a Q block size -- `blk` of sage_quant_int8 when it quantises Q, `blkq`
+ * of sage_attn_fwd, sage_attn_fwd_masked, sage_sageattn*, sage_sageattn_workspace_bytes -- it gives every block of blkq
+ * rows EIGHT scales instead of one: scale g of a block covers the rows r of the block with r % 8 == g, and the scale
+ * tensor holds ceil(S/blkq)*8 values per head, scale[(b*H + h)*ceil(S/blkq)*8 + block*8 + g].  This is the granularity
+ * upstream SageAttention calls per-thread (its WARPQ = blkq: on its MMA fragments the rows i, i+8, i+16, ... of a
+ * warp tile sit in one thread; here a query row is a lane of the transposed score tile, so a scale per row group costs
+ * nothing extra in the kernel).  The reference names it as a finer granularity next to the (128, 16, -1, 1) recipe of
+ * backends/_mthreads/docs/sageAttention_mthread.md:36-42 and has no code for it: the quantiser arithmetic is that of
+ * quant_per_block.py:38-46 applied per row group.  Fixed-length batches only; not for K; the Q quantisation fused into the
+ * attention kernel (sage_attn_fwd_qfused) does not take it -- sage_sageattn* run the standalone Q pass instead. */
+#define SAGE_BLK_INTERLEAVE8 0x100
+
 /* Rows of K/V covered by one V panel (see sage_prep_v). */
 #define SAGE_PANEL_ROWS 128
 
@@ -66,7 +78,8 @@ const char* sage_last_error(void);
  * scale:  fp32; fixed-length: scale[(b*H + h)*ceil(L/blk) + block];
  *         packed: scale[h*scale_sh + cu_blocks[b] + block] (cu_blocks from sage_varlen_plan).
  * mult:   sm_scale*1.44269504 for Q (quant_per_block.py:87), 1.0 for K (:97).
- * blk in {16,32,64,128}; D in {64,128}.  In packed mode L is the longest sequence.
+ * blk in {16,32,64,128}, optionally | SAGE_BLK_INTERLEAVE8 (Q only, fixed-length only); D in {64,128}.  In packed mode L
+ * is the longest sequence.
  */
 int sage_quant_int8(const void* x, int8_t* out, float* scale, const void* km,
                     int B, int H, int L, int D,

@@ -8,6 +8,8 @@ Reference lines followed:
   * kernel   backends/_enflame/ops/sage_attention/quant_per_block.py:20-46
   * host     backends/_enflame/ops/sage_attention/quant_per_block.py:49-101
   * guard    backends/_hygon/ops/sageattention/sageattention_triton.py:35
+Parity unpinned (not in the reference's code, defined here and pinned against the mathematics in the tests): k_mean,
+quant_v_fp8, and the eight interleaved scales per block of quant_per_block_int8(groups=8).
 """
 from __future__ import annotations
 
@@ -46,11 +48,15 @@ def quant_tile_int8(x32: np.ndarray, mult) -> tuple[np.ndarray, np.float32]:
     return q, np.float32(scale)
 
 
-def quant_per_block_int8(x_hnd32: np.ndarray, blk: int, mult) -> tuple[np.ndarray, np.ndarray]:
-    """[B, H, L, C] float32 -> (int8 [B,H,L,C], float32 scale [B,H,ceil(L/blk)]).
+def quant_per_block_int8(x_hnd32: np.ndarray, blk: int, mult, groups: int = 1) -> tuple[np.ndarray, np.ndarray]:
+    """[B, H, L, C] float32 -> (int8 [B,H,L,C], float32 scale [B,H,ceil(L/blk)*groups]).
 
     Vectorised over tiles; identical arithmetic to ``quant_tile_int8``.
     Grid of quant_per_block.py:81 / :91: one program per (block, head, batch).
+    ``groups`` = 8: eight interleaved scales per block, scale g for the rows r of the block with r % 8 == g (the
+    granularity upstream SageAttention calls per-thread, with its WARPQ = blk).  The reference has no code for it
+    (parity unpinned): it is defined here as the same tile arithmetic applied to each row group, and pinned in the
+    tests against a row-by-row loop over ``quant_tile_int8``.
     """
     B, H, L, C = x_hnd32.shape
     nblk = (L + blk - 1) // blk
@@ -58,13 +64,14 @@ def quant_per_block_int8(x_hnd32: np.ndarray, blk: int, mult) -> tuple[np.ndarra
     x = x_hnd32.astype(np.float32, copy=False) * np.float32(mult)
     if pad:
         x = np.concatenate([x, np.zeros((B, H, pad, C), np.float32)], axis=2)
-    xt = x.reshape(B, H, nblk, blk * C)
-    amax = np.max(np.abs(xt), axis=-1).astype(np.float32)
-    scale = np.maximum(amax / np.float32(127.0), SCALE_FLOOR).astype(np.float32)
-    z = xt / scale[..., None]
+    # [.., block, row group member, group, channel]: with groups == 1 a block is one group of blk rows
+    xt = x.reshape(B, H, nblk, blk // groups, groups, C)
+    amax = np.max(np.abs(xt), axis=(3, 5)).astype(np.float32)
+    scale = np.maximum(amax / np.float32(127.0), SCALE_FLOOR).astype(np.float32)          # [B, H, nblk, groups]
+    z = xt / scale[:, :, :, None, :, None]
     z = z + np.float32(0.5) * np.where(z >= 0, np.float32(1.0), np.float32(-1.0)).astype(np.float32)
     q = np.trunc(z).astype(np.int32).astype(np.int8).reshape(B, H, nblk * blk, C)[:, :, :L]
-    return np.ascontiguousarray(q), scale
+    return np.ascontiguousarray(q), np.ascontiguousarray(scale.reshape(B, H, nblk * groups))
 
 
 def _hnd(x: np.ndarray, layout: str) -> np.ndarray:
@@ -83,18 +90,19 @@ def q_multiplier(head_dim: int, sm_scale=None) -> np.float32:
     return np.float32(float(sm_scale) * LOG2E_REF)
 
 
-def per_block_int8(q, k, km=None, BLKQ=128, BLKK=64, sm_scale=None, tensor_layout="HND"):
+def per_block_int8(q, k, km=None, BLKQ=128, BLKK=64, sm_scale=None, tensor_layout="HND", q_interleave=1):
     """Restates per_block_int8 (quant_per_block.py:49-101) on CPU tensors.
 
     Returns torch CPU tensors (q_int8, q_scale, k_int8, k_scale) with the reference's
-    shapes: int8 like q / k, scales [B, H, ceil(L/BLK)] float32.
+    shapes: int8 like q / k, scales [B, H, ceil(L/BLK)] float32 (q_scale [B, H, ceil(L/BLKQ)*8] with
+    ``q_interleave=8``, see quant_per_block_int8).
     """
     if km is not None:
         k = k - km  # input-dtype subtraction, quant_per_block.py:53-54
     q32 = _hnd(_to_f32(q), tensor_layout)
     k32 = _hnd(_to_f32(k), tensor_layout)
     head_dim = q32.shape[-1]
-    qi, qs = quant_per_block_int8(q32, BLKQ, q_multiplier(head_dim, sm_scale))
+    qi, qs = quant_per_block_int8(q32, BLKQ, q_multiplier(head_dim, sm_scale), q_interleave)
     ki, ks = quant_per_block_int8(k32, BLKK, np.float32(1.0))
     qi = np.ascontiguousarray(_hnd(qi, tensor_layout)) if tensor_layout == "NHD" else qi
     ki = np.ascontiguousarray(_hnd(ki, tensor_layout)) if tensor_layout == "NHD" else ki

@@ -39,6 +39,10 @@ def test_size_queries_do_not_need_a_gpu(sage_lib):
     assert sage_lib.sage_v_panel_bytes(1, 24, 32760, 128, _cabi.PV_FP16) == 24 * 256 * 128 * 128 * 2
     assert sage_lib.sage_k_mean_workspace_bytes(2, 32, 16384, 128) >= 2 * 32 * 32 * 128 * 8
     assert sage_lib.sage_sageattn_workspace_bytes(2, 32, 32, 16384, 16384, 128, 64, 128, 1, 0, 0, 0) > 3 * 2 * 32 * 16384 * 128
+    # eight interleaved Q scales per block: seven more floats per (batch, head, block)
+    a = sage_lib.sage_sageattn_workspace_bytes(1, 4, 4, 4096, 4096, 128, 32, 64, 1, 0, 0, 0)
+    b = sage_lib.sage_sageattn_workspace_bytes(1, 4, 4, 4096, 4096, 128, 32 | 0x100, 64, 1, 0, 0, 0)
+    assert b - a == 4 * 128 * 7 * 4
     n = sage_lib.sage_varlen_plan_ints(16, 266000)
     offs = (ctypes.c_int64 * 5)()
     sage_lib.sage_varlen_plan_offsets(16, 266000, offs)
@@ -81,6 +85,13 @@ def test_attn_argument_errors(sage_lib):
     assert call(blkq=8) == _cabi.SAGE_ENOTIMPL       # Q scale blocks: 16, 32, 64 or 128 rows
     assert call(pv=1) == _cabi.SAGE_EINVAL           # fp8 needs v_scale
     assert call(pv=5) == _cabi.SAGE_EINVAL
+    # interleaved Q scales (SAGE_BLK_INTERLEAVE8 = 0x100 OR-ed into blkq): a Q granularity of fixed-length batches
+    assert call(blkk=64 | 0x100) == _cabi.SAGE_ENOTIMPL
+    assert call(blkq=8 | 0x100) == _cabi.SAGE_ENOTIMPL
+    rc = sage_lib.sage_attn_fwd(FAKE, FAKE, FAKE, FAKE, FAKE, NULL, FAKE, NULL, 1, 4, 2, 128, 128, 128,
+                                0, 128 * 128, 128, 0, 128 * 128, 128, 0, 128 * 128, 128, 32 | 0x100, 64, 0, 0, 0,
+                                FAKE, FAKE, FAKE, 128, 0, 0, 0, NULL)
+    assert rc == _cabi.SAGE_ENOTIMPL and "packed" in sage_lib.sage_last_error().decode()
 
 
 def test_attn_alignment_and_slice_limits(sage_lib):

@@ -281,6 +281,74 @@ def test_q_scale_blocks_of_16_rows(pv, causal):
 
 
 @pytest.mark.parametrize("layout", ["HND", "NHD"])
+@pytest.mark.parametrize("pv", ["fp16", "fp8"])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("blkq,D", [(32, 128), (128, 128), (16, 64), (64, 64)])
+def test_interleaved_q_scales(layout, pv, causal, blkq, D):
+    """Eight interleaved Q scales per block (rows r, r+8, ... share one; upstream's per-thread granularity, no code in
+    the reference): `forward` on such operands against the reference formula with the scales expanded row by row,
+    GQA, ragged lengths, LSE; and the one-call pipeline, which must equal quantise-then-forward bit for bit."""
+    g = torch.Generator().manual_seed(808 + blkq + D + int(causal))
+    B, Hq, Hkv, Sq, Skv = 2, 4, 2, 301, 301 if causal else 215
+    q = randn(layout, B, Hq, Sq, D, torch.float16, g)
+    k = randn(layout, B, Hkv, Skv, D, torch.float16, g)
+    v = randn(layout, B, Hkv, Skv, D, torch.float16, g)
+    (q if layout == "HND" else q.transpose(1, 2))[1, 2, 77] *= 25.0      # an outlier row: only its own group pays for it
+    qd, kd, vd = q.to(DEV), k.to(DEV), v.to(DEV)
+    qi, qs, ki, ks = sa.per_block_int8(qd, kd, BLKQ=blkq, BLKK=64, tensor_layout=layout, q_interleave=8)
+    assert tuple(qs.shape) == (B, Hq, (Sq + blkq - 1) // blkq * 8)
+    out, lse = sa.forward(qi, ki, vd, qs, ks, tensor_layout=layout, return_lse=True, BLKQ=blkq, BLKK=64, is_causal=causal,
+                          pv_mode=pv, q_interleave=8)
+    torch.cuda.synchronize()
+    ref, ref_lse = oa.sage_reference(qi.cpu(), ki.cpu(), v, qs.cpu(), ks.cpu(), layout, blkq, 64, is_causal=causal,
+                                     q_interleave=8)
+    m = oa.metrics(out.cpu().float(), ref)
+    assert m["finite"] and (m["rel_rmse"] < 2e-3 if pv == "fp16" else (m["cosine"] >= 0.999 and m["rel_rmse"] < 5e-2)), m
+    # (the reference's own bound on LSE2 is 3e-2, test_sageattention_hip.py:52-58; the outlier row's logits are 25 times larger)
+    assert (lse.cpu().double() - ref_lse).abs().max().item() < (5e-3 if pv == "fp16" else 3e-2)
+    # a q_scale of the per-block shape is refused, and so is the keyword's absence for an interleaved one
+    with pytest.raises(ValueError):
+        sa.forward(qi, ki, vd, qs, ks, tensor_layout=layout, BLKQ=blkq, BLKK=64, pv_mode=pv)
+    # the finer scales are at least as accurate as one scale per block on the outlier's neighbours
+    qi1, qs1, _, _ = sa.per_block_int8(qd, kd, BLKQ=blkq, BLKK=64, tensor_layout=layout)
+    out1, _ = sa.forward(qi1, ki, vd, qs1, ks, tensor_layout=layout, BLKQ=blkq, BLKK=64, is_causal=causal, pv_mode="fp16")
+    out8, _ = sa.forward(qi, ki, vd, qs, ks, tensor_layout=layout, BLKQ=blkq, BLKK=64, is_causal=causal, pv_mode="fp16",
+                         q_interleave=8)
+    exact = oa.sdpa_fp32(q, k, v, layout, causal)
+    e1 = oa.metrics(out1.cpu().float(), exact)["rmse"]
+    e8 = oa.metrics(out8.cpu().float(), exact)["rmse"]
+    assert e8 <= e1 * 1.02, (e1, e8)
+    # one call: standalone Q pass inside, same result as the two steps (no K smoothing so that K is the same tensor)
+    one = sa.sageattn(qd, kd, vd, tensor_layout=layout, is_causal=causal, smooth_k=False, pv_mode=pv, BLKQ=blkq, BLKK=64,
+                      q_interleave=8)
+    two, _ = sa.forward(qi, ki, vd, qs, ks, tensor_layout=layout, BLKQ=blkq, BLKK=64, is_causal=causal, pv_mode=pv,
+                        q_interleave=8, output_dtype=torch.float16)
+    assert torch.equal(one, two)
+
+
+def test_interleaved_q_scales_with_mask_lse_and_smoothing_against_fp32_sdpa():
+    """sageattn(q_interleave=8) with K smoothing, LSE and an additive mask: against FP32 SDPA on the raw inputs."""
+    g = torch.Generator().manual_seed(909)
+    B, Hq, Hkv, S, D = 1, 4, 2, 260, 128
+    q = randn("HND", B, Hq, S, D, torch.bfloat16, g)
+    k = randn("HND", B, Hkv, S, D, torch.bfloat16, g, offset_std=2.0)
+    v = randn("HND", B, Hkv, S, D, torch.bfloat16, g)
+    mask = (torch.randn((1, 1, S, S), generator=g) * 0.5).float()
+    out, lse = sa.sageattn(q.to(DEV), k.to(DEV), v.to(DEV), attn_mask=mask.to(DEV), return_lse=True, BLKQ=32, BLKK=64,
+                           q_interleave=8)
+    qq, kk, vv = q.double(), k.double().repeat_interleave(2, 1), v.double().repeat_interleave(2, 1)
+    logits = qq @ kk.transpose(-1, -2) * D ** -0.5 + mask.double()
+    ref = torch.softmax(logits, -1) @ vv
+    m = oa.metrics(out.cpu().float(), ref)
+    assert m["finite"] and m["cosine"] >= 0.999, m
+    assert (lse.cpu().double() - torch.logsumexp(logits, -1)).abs().max().item() < 3e-2
+    with pytest.raises(NotImplementedError):
+        cu = torch.tensor([0, 100, 260], dtype=torch.int32, device=DEV)
+        sa.sageattn(q[0].transpose(0, 1).contiguous().to(DEV), k[0].transpose(0, 1).contiguous().to(DEV),
+                    v[0].transpose(0, 1).contiguous().to(DEV), cu_seqlens_q=cu, cu_seqlens_k=cu, q_interleave=8)
+
+
+@pytest.mark.parametrize("layout", ["HND", "NHD"])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("cfg", [(128, 64, "fp16", False, 64), (64, 128, "fp8", True, 128), (32, 32, "fp8", False, 128),
                                  (128, 128, "fp16", True, 128)])

@@ -24,6 +24,31 @@ def _cmp(q, k, km=None, layout="HND", BLKQ=128, BLKK=64, sm_scale=None):
     return out
 
 
+@pytest.mark.parametrize("layout", ["HND", "NHD"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("BLKQ", [16, 32, 64, 128])
+def test_interleaved_q_scales_bit_exact(layout, dtype, D, BLKQ):
+    """Eight interleaved scales per Q block (rows r with r % 8 == g share scale g): int8 values and scales equal the
+    oracle's bit for bit, ragged last block, outlier rows and all-zero groups included."""
+    g = torch.Generator().manual_seed(77 + D + BLKQ)
+    q = randn(layout, 2, 3, 301, D, dtype, g)
+    k = randn(layout, 2, 3, 70, D, dtype, g)
+    qv = q if layout == "HND" else q.transpose(1, 2)
+    qv[0, 1, 37] *= 30.0
+    qv[1, 2, 256:264] = 0.0
+    qv[1, 0, 300] = 0.0
+    out = sa.per_block_int8(q.to(DEV), k.to(DEV), BLKQ=BLKQ, BLKK=64, sm_scale=0.2, tensor_layout=layout, q_interleave=8)
+    ref = oq.per_block_int8(q, k, BLKQ=BLKQ, BLKK=64, sm_scale=0.2, tensor_layout=layout, q_interleave=8)
+    torch.cuda.synchronize()
+    assert tuple(out[1].shape) == (2, 3, (301 + BLKQ - 1) // BLKQ * 8)
+    for name, a, b in zip(("q_int8", "q_scale", "k_int8", "k_scale"), out, ref):
+        assert a.dtype == b.dtype and tuple(a.shape) == tuple(b.shape), name
+        assert torch.equal(a.cpu(), b), f"{name}: {(a.cpu() != b).sum().item()} mismatches"
+    with pytest.raises(ValueError):
+        sa.per_block_int8(q.to(DEV), k.to(DEV), q_interleave=4)
+
+
 def test_reference_golden_vectors(golden):
     for name in golden["cases"]:
         c = golden_case(golden, str(name))

@@ -196,3 +196,34 @@ def test_varlen_equals_per_sequence():
     assert offq.tolist() == [0, 1, 3, 5, 6]
     a, b, c, d = oq.per_block_int8(q[70:199].unsqueeze(0), k[70:199].unsqueeze(0), tensor_layout="NHD")
     assert torch.equal(qi[70:199], a[0]) and torch.equal(qs[:, 1:3], b[0])
+
+
+def test_interleaved_q_scales_equal_the_tile_quantiser_applied_to_each_row_group():
+    """Eight interleaved scales per block (the granularity upstream SageAttention calls per-thread; no code in the
+    reference: parity unpinned): by definition the tile arithmetic of quant_per_block.py:38-46 on the rows r of a block
+    with r % 8 == g.  The vectorised oracle is pinned against that row-group loop, ragged last block and empty groups
+    included, and with one group it is the per-block quantiser."""
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((2, 3, 70, 64)).astype(np.float32) * np.float32(3.0)
+    x[0, 1, 33] *= np.float32(40.0)                       # an outlier row only raises the scale of its own group
+    for blk in (16, 32, 64, 128):
+        q1, s1 = oq.quant_per_block_int8(x, blk, 0.3)
+        q1b, s1b = oq.quant_per_block_int8(x, blk, 0.3, 1)
+        assert np.array_equal(q1, q1b) and np.array_equal(s1, s1b)
+        q8, s8 = oq.quant_per_block_int8(x, blk, 0.3, 8)
+        nblk = (70 + blk - 1) // blk
+        assert s8.shape == (2, 3, nblk * 8) and q8.shape == x.shape
+        for b in range(2):
+            for h in range(3):
+                for t in range(nblk):
+                    for g in range(8):
+                        rows = [r for r in range(t * blk, min(70, (t + 1) * blk)) if r % 8 == g]
+                        if not rows:
+                            assert s8[b, h, t * 8 + g] == oq.SCALE_FLOOR
+                            continue
+                        qq, ss = oq.quant_tile_int8(x[b, h, rows], 0.3)
+                        assert ss == s8[b, h, t * 8 + g] and np.array_equal(qq, q8[b, h, rows]), (blk, b, h, t, g)
+    _, s8 = oq.quant_per_block_int8(x, 32, 0.3, 8)
+    _, s1 = oq.quant_per_block_int8(x, 32, 0.3)
+    assert s8[0, 1, 8 + 1] == s1[0, 1, 1] and (s8[0, 1, 8:16] <= s1[0, 1, 1]).all() and s8[0, 1, 8] < 0.2 * s1[0, 1, 1]
+
