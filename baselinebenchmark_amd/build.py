@@ -14,7 +14,8 @@ from pathlib import Path
 
 CSRC = Path(__file__).resolve().parent / "csrc"
 LIB = CSRC / "libsage_mi355x.so"
-SOURCES = ["sage_quant.hip", "sage_attn.hip", "sage_attn_mask.hip", "sage_attn_qfuse.hip", "sage_api.hip", "sage_static.hip"]
+SOURCES = ["sage_quant.hip", "sage_attn.hip", "sage_attn_mask.hip", "sage_attn_qfuse.hip", "sage_attn_kinterleave.hip", "sage_api.hip",
+           "sage_static.hip"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     # correctly rounded fp32 divide (the INT8 quantiser's contract) and no packed-fp32 selection

@@ -35,8 +35,13 @@ bool valid_blk_attn(int blk) { return blk == 16 || blk == 32 || blk == 64 || blk
 bool valid_blkk_attn(int blk) { return valid_blk_attn(blk); }
 int ilog2(int x) { int r = 0; while ((1 << r) < x) r++; return r; }
 // A Q block-size argument may carry SAGE_BLK_INTERLEAVE8: eight interleaved scales per block instead of one.
-int blk_rows(int blk) { return blk > 0 ? (blk & ~SAGE_BLK_INTERLEAVE8) : blk; }
-int blk_groups(int blk) { return (blk > 0 && (blk & SAGE_BLK_INTERLEAVE8)) ? 8 : 1; }
+// ... or SAGE_BLK_INTERLEAVE4 (a K block size): four.  Both flags at once decode to 0 groups, which nothing accepts.
+int blk_rows(int blk) { return blk > 0 ? (blk & ~(SAGE_BLK_INTERLEAVE8 | SAGE_BLK_INTERLEAVE4)) : blk; }
+int blk_groups(int blk) {
+  if (blk <= 0) return 1;
+  const bool g8 = blk & SAGE_BLK_INTERLEAVE8, g4 = blk & SAGE_BLK_INTERLEAVE4;
+  return g8 && g4 ? 0 : g8 ? 8 : g4 ? 4 : 1;
+}
 
 int check_common(int B, int H, int L, int D, int dtype) {
   if (B < 0 || H < 0 || L < 0) return fail(SAGE_EINVAL, "negative dimension (B=%d H=%d L=%d)", B, H, L);
@@ -82,8 +87,9 @@ int quant_impl(const void* x, int8_t* out, float* scale, const void* km, int B, 
   const int groups = blk_groups(blk);
   blk = blk_rows(blk);
   if (!valid_blk_quant(blk)) return fail(SAGE_ENOTIMPL, "quantisation block %d is not supported (16, 32, 64, 128)", blk);
+  if (groups == 0) return fail(SAGE_EINVAL, "SAGE_BLK_INTERLEAVE8 and SAGE_BLK_INTERLEAVE4 exclude each other");
   if (groups > 1 && cu_seqlens) return fail(SAGE_ENOTIMPL, "interleaved scales are not supported for packed batches");
-  if (groups > 1 && km) return fail(SAGE_ENOTIMPL, "interleaved scales are a Q granularity: not together with a K mean");
+  if (groups == 4 && blk == 16) return fail(SAGE_ENOTIMPL, "four interleaved scales need blocks of 32, 64 or 128 rows");
   if (B == 0 || H == 0 || L == 0) return SAGE_OK;
   if (!x || !out || !scale) return fail(SAGE_EINVAL, "null tensor pointer");
   if (cu_seqlens && !cu_blocks) return fail(SAGE_EINVAL, "packed mode needs cu_blocks");
@@ -220,12 +226,17 @@ int attn_impl(const int8_t* q, const int8_t* k, const void* v_panels, const floa
   if (Hkv <= 0 || Hq % Hkv) return fail(SAGE_EINVAL, "query heads (%d) must be divisible by KV heads (%d)", Hq, Hkv);
   if (Skv < 0) return fail(SAGE_EINVAL, "negative kv length");
   if (pv_mode != SAGE_PV_FP16 && pv_mode != SAGE_PV_FP8) return fail(SAGE_EINVAL, "pv_mode %d unknown", pv_mode);
-  const int qgroups = blk_groups(blkq);
+  const int qgroups = blk_groups(blkq), kgroups = blk_groups(blkk);
   blkq = blk_rows(blkq);
+  blkk = blk_rows(blkk);
   if (!valid_blk_attn(blkq) || !valid_blkk_attn(blkk))
     return fail(SAGE_ENOTIMPL, "attention needs Q and K scale blocks of 16, 32, 64 or 128 rows (got %d/%d)", blkq, blkk);
-  if (qgroups > 1 && cu_seqlens_q) return fail(SAGE_ENOTIMPL, "interleaved Q scales are not supported for packed batches");
+  if ((qgroups != 1 && qgroups != 8) || (kgroups != 1 && kgroups != 4))
+    return fail(SAGE_ENOTIMPL, "Q scale blocks take SAGE_BLK_INTERLEAVE8, K scale blocks SAGE_BLK_INTERLEAVE4");
+  if ((qgroups > 1 || kgroups > 1) && cu_seqlens_q) return fail(SAGE_ENOTIMPL, "interleaved scales are not supported for packed batches");
   if (qgroups > 1 && qraw.ptr) return fail(SAGE_ENOTIMPL, "interleaved Q scales need the standalone Q quantiser (sage_quant_int8)");
+  if (kgroups > 1 && blkk == 16) return fail(SAGE_ENOTIMPL, "interleaved K scales need blocks of 32, 64 or 128 keys");
+  if (kgroups > 1 && mask.ptr) return fail(SAGE_ENOTIMPL, "interleaved K scales cannot be combined with an explicit mask");
   if (blkk == 16 && mask.ptr) return fail(SAGE_ENOTIMPL, "K scale blocks of 16 rows cannot be combined with an explicit mask");
   if (B == 0 || Hq == 0 || Sq == 0) return SAGE_OK;
   if (!out || (Skv > 0 && (!k || !v_panels || !k_scale))) return fail(SAGE_EINVAL, "null tensor pointer");
@@ -256,7 +267,7 @@ int attn_impl(const int8_t* q, const int8_t* k, const void* v_panels, const floa
   a.B = B; a.Hq = Hq; a.Hkv = Hkv; a.Sq = Sq; a.Skv = Skv;
   a.q_sb = q_sb; a.q_sh = q_sh; a.q_sn = q_sn; a.k_sb = k_sb; a.k_sh = k_sh; a.k_sn = k_sn;
   a.o_sb = o_sb; a.o_sh = o_sh; a.o_sn = o_sn;
-  a.blkq = blkq; a.blkk = blkk; a.blkq_shift = ilog2(blkq); a.blkk_shift = ilog2(blkk); a.qg_shift = qgroups == 8 ? 3 : 0;
+  a.blkq = blkq; a.blkk = blkk; a.blkq_shift = ilog2(blkq); a.blkk_shift = ilog2(blkk); a.qg_shift = qgroups == 8 ? 3 : 0; a.k_interleave = kgroups == 4;
   a.out_bf16 = out_dtype == SAGE_DT_BF16;
   a.nqt = (Sq + BM - 1) / BM;
   a.mask = mask.ptr; a.mask_kind = mask.kind; a.m_sb = mask.sb; a.m_sh = mask.sh; a.m_sm = mask.sm; a.m_sn = mask.sn;
@@ -334,13 +345,13 @@ E2EWorkspace e2e_layout(int B, int Hq, int Hkv, int Sq, int Skv, int D, int blkq
   w.q_i8 = off; off += align_up(nq);
   w.k_i8 = off; off += align_up(nk);
   if (varlen) {
-    w.qs_sh = total_q / blk_rows(blkq) + B; w.ks_sh = total_k / blkk + B; w.panel_sh = total_k / SAGE_PANEL_ROWS + B;
+    w.qs_sh = total_q / blk_rows(blkq) + B; w.ks_sh = total_k / blk_rows(blkk) + B; w.panel_sh = total_k / SAGE_PANEL_ROWS + B;
     w.q_scale = off; off += align_up((size_t)Hq * w.qs_sh * 4);
     w.k_scale = off; off += align_up((size_t)Hkv * w.ks_sh * 4);
   } else {
     w.qs_sh = w.ks_sh = w.panel_sh = 0;
     w.q_scale = off; off += align_up((size_t)B * Hq * ((Sq + blk_rows(blkq) - 1) / blk_rows(blkq)) * blk_groups(blkq) * 4);
-    w.k_scale = off; off += align_up((size_t)B * Hkv * ((Skv + blkk - 1) / blkk) * 4);
+    w.k_scale = off; off += align_up((size_t)B * Hkv * ((Skv + blk_rows(blkk) - 1) / blk_rows(blkk)) * (blk_groups(blkk) ? blk_groups(blkk) : 1) * 4);
   }
   w.km = off; off += align_up((size_t)B * Hkv * D * 2);
   w.v_scale = off; off += align_up((size_t)B * Hkv * D * 4);
@@ -381,11 +392,15 @@ int sage_sageattn_masked(const void* q, const void* k, const void* v, void* out,
                          int64_t m_sm, int64_t m_sn, sage_stream_t stream) {
   if (int rc = check_common(B, Hq, Sq, D, dtype)) return rc;
   if (Hkv <= 0 || Hq % Hkv) return fail(SAGE_EINVAL, "query heads (%d) must be divisible by KV heads (%d)", Hq, Hkv);
-  if (!valid_blk_attn(blk_rows(blkq)) || !valid_blkk_attn(blkk))
-    return fail(SAGE_ENOTIMPL, "Q and K scale blocks must be 16, 32, 64 or 128 rows (got %d/%d)", blk_rows(blkq), blkk);
+  if (!valid_blk_attn(blk_rows(blkq)) || !valid_blkk_attn(blk_rows(blkk)))
+    return fail(SAGE_ENOTIMPL, "Q and K scale blocks must be 16, 32, 64 or 128 rows (got %d/%d)", blk_rows(blkq), blk_rows(blkk));
+  if ((blk_groups(blkq) != 1 && blk_groups(blkq) != 8) || (blk_groups(blkk) != 1 && blk_groups(blkk) != 4))
+    return fail(SAGE_ENOTIMPL, "Q scale blocks take SAGE_BLK_INTERLEAVE8, K scale blocks SAGE_BLK_INTERLEAVE4");
+  if (blk_groups(blkk) == 4 && (blk_rows(blkk) == 16 || attn_mask))
+    return fail(SAGE_ENOTIMPL, "interleaved K scales need blocks of 32, 64 or 128 keys and no explicit mask");
   if (pv_mode != SAGE_PV_FP16 && pv_mode != SAGE_PV_FP8) return fail(SAGE_EINVAL, "pv_mode %d unknown", pv_mode);
   const int varlen = cu_seqlens_q != nullptr;
-  if (varlen && blk_groups(blkq) > 1) return fail(SAGE_ENOTIMPL, "interleaved Q scales are not supported for packed batches");
+  if (varlen && (blk_groups(blkq) > 1 || blk_groups(blkk) > 1)) return fail(SAGE_ENOTIMPL, "interleaved scales are not supported for packed batches");
   if (varlen && !cu_seqlens_k) return fail(SAGE_EINVAL, "packed mode needs cu_seqlens_k");
   if (B == 0 || Hq == 0 || Sq == 0) return SAGE_OK;
   if (!workspace) return fail(SAGE_EWORKSPACE, "null workspace");

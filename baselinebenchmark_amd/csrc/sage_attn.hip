@@ -130,6 +130,7 @@ AttnConfig attn_config(int D, int pv, bool packed) {
 hipError_t launch_attn(const AttnArgs& a, int D, int pv, bool causal, int grid, hipStream_t st) {
   if (grid == 0) return hipSuccess;
   if (a.mask) return launch_attn_masked(a, D, pv, grid, st);
+  if (a.k_interleave) return launch_attn_kinterleaved(a, D, pv, causal, grid, st);
   if (a.blkk == 16) return launch_attn_k16(a, D, pv, causal, grid, st);
   if (a.q_raw) return launch_attn_qfused(a, D, pv, causal, grid, st);
   const bool msum = pv && a.lse == nullptr;   // row sums on the matrix pipe unless LSE is wanted

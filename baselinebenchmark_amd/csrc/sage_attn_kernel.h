@@ -146,7 +146,8 @@ static __device__ unsigned long long g_tile_timing[kTimingSets][48];
 #endif
 // MASK: 0 none, 1 boolean keep-mask (bytes), 2 additive fp32 bias in base-2 score units
 // (sageattention_triton.py:92-105), both [B, Hq, Sq, Skv] with element strides.
-// KSUB: K scale blocks per 32 keys (1 for blocks of 32/64/128 keys, 2 for blocks of 16 keys).
+// KSUB: K scale blocks per 32 keys (1 for blocks of 32/64/128 keys, 2 for blocks of 16 keys); 3 = four interleaved scales per
+// block of 32/64/128 keys, scale t for the keys n of the block with (n % 8) / 2 == t (two of them reach every lane).
 // QF: the kernel reads fp16/bf16 Q and quantises its own tile (same arithmetic as quant_int8_kernel).
 template <int D, int NW, int BN, int PV, bool CAUSAL, bool MSUM, int MASK, int KSUB = 1, bool QF = false>
 __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
@@ -255,7 +256,7 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
     koff = (int64_t)b * a.k_sb + (int64_t)kvh * a.k_sh;
     lseoff = ((int64_t)b * a.Hq + hq) * a.Sq;
     qsp = a.qs + (((int64_t)b * a.Hq + hq) * ((Lq + a.blkq - 1) / a.blkq) << a.qg_shift);
-    ksp = a.ks + ((int64_t)b * a.Hkv + kvh) * ((Lk + a.blkk - 1) / a.blkk);
+    ksp = a.ks + ((int64_t)b * a.Hkv + kvh) * ((Lk + a.blkk - 1) / a.blkk) * (KSUB == 3 ? 4 : 1);
     vbase = a.vp + ((int64_t)b * a.Hkv + kvh) * ((Lk + kPanelRows - 1) / kPanelRows) * PANEL_BYTES;
   }
   nkblk = (Lk + a.blkk - 1) / a.blkk;
@@ -466,9 +467,23 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
   v16i acc[NT];
   // q_scale * k_scale per K scale block of the tile; in the accumulator layout register r of a 32-key
   // group holds keys 8*(r/4) + 4*h + r%4, so registers 0-7 belong to the first 16 keys and 8-15 to the rest.
-  constexpr int NSC = NT * KSUB;
+  // With interleaved K scales (KSUB == 3) a key's scale is picked by (n % 8) / 2 = 2*h + (r % 4) / 2: two per lane and
+  // 32-key group, selected by bit 1 of the register index.
+  constexpr int SUBS = KSUB == 1 ? 1 : 2;   // scale values per 32-key group and lane
+  constexpr int NSC = NT * SUBS;
   float sc[NSC];
-  auto sci = [](int nt, int r) { return KSUB == 2 ? 2 * nt + r / 8 : nt; };
+  auto subof = [](int r) { return KSUB == 2 ? r / 8 : KSUB == 3 ? (r >> 1) & 1 : 0; };
+  auto sci = [&](int nt, int r) { return SUBS * nt + subof(r); };
+  // K scale i of tile j as this lane needs it (before the Q scale is multiplied in)
+  auto kscale_at = [&](int j, int i) -> float {
+    if constexpr (KSUB == 3) {
+      const int blk = min((j * BN + 32 * (i >> 1)) >> a.blkk_shift, nkblk - 1);
+      const float lo = ksc[blk * 4 + (i & 1)], hi = ksc[blk * 4 + 2 + (i & 1)];
+      return h ? hi : lo;
+    } else {
+      return ksc[min((j * BN + (32 / KSUB) * i) >> a.blkk_shift, nkblk - 1)];
+    }
+  };
   float mloc = kNegInf;
 
   // ---- S^T = K . Q^T (int8 -> int32 on the biased accumulators), then mask and row maximum ----
@@ -504,7 +519,7 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
   // load in flight while K/V fragments are being read would force every LDS wait to drain the queue.
   auto load_scales = [&](int j) {
 #pragma unroll
-    for (int i = 0; i < NSC; i++) sc[i] = qscale * ksc[min((j * BN + (32 / KSUB) * i) >> a.blkk_shift, nkblk - 1)];
+    for (int i = 0; i < NSC; i++) sc[i] = qscale * kscale_at(j, i);
   };
 
   auto rowmax = [&](int j) {
@@ -552,12 +567,20 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
 #pragma unroll
     for (int nt = 0; nt < NT; nt++) {
 #pragma unroll
-      for (int sub = 0; sub < KSUB; sub++) {
-        constexpr int RS = 16 / KSUB;
-        int mx = acc[nt][sub * RS];
+      for (int sub = 0; sub < SUBS; sub++) {
+        if constexpr (KSUB == 3) {
+          int mx = acc[nt][2 * sub];
 #pragma unroll
-        for (int r = 1; r < RS; r++) mx = max(mx, acc[nt][sub * RS + r]);
-        mloc = fmaxf(mloc, __builtin_fmaf(as_f(mx), sc[nt * KSUB + sub], -kBiasF * sc[nt * KSUB + sub]));
+          for (int r = 1; r < 16; r++)
+            if (subof(r) == sub && r != 2 * sub) mx = max(mx, acc[nt][r]);
+          mloc = fmaxf(mloc, __builtin_fmaf(as_f(mx), sc[nt * SUBS + sub], -kBiasF * sc[nt * SUBS + sub]));
+        } else {
+          constexpr int RS = 16 / KSUB;
+          int mx = acc[nt][sub * RS];
+#pragma unroll
+          for (int r = 1; r < RS; r++) mx = max(mx, acc[nt][sub * RS + r]);
+          mloc = fmaxf(mloc, __builtin_fmaf(as_f(mx), sc[nt * KSUB + sub], -kBiasF * sc[nt * KSUB + sub]));
+        }
       }
     }
   };
@@ -567,7 +590,7 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
     // next tile's K scales: requested first, consumed last
     float kraw[NSC];
 #pragma unroll
-    for (int i = 0; i < NSC; i++) kraw[i] = ksc[min(((j + 1) * BN + (32 / KSUB) * i) >> a.blkk_shift, nkblk - 1)];
+    for (int i = 0; i < NSC; i++) kraw[i] = kscale_at(j + 1, i);
     const float mall = xchg32_max(mloc);
     // lazy rescale: move the reference maximum only when it grew by more than TAU
     if (__builtin_amdgcn_ballot_w64(mall > m_used + TAU) != 0) {
@@ -597,15 +620,15 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
       const float k0 = 8.0f * (PSHIFT - m_used) + (56.0f + kCodeBias);
 #pragma unroll
       for (int nt = 0; nt < NT; nt++) {
-        float c[KSUB], mul[KSUB];
+        float c[SUBS], mul[SUBS];
 #pragma unroll
-        for (int sub = 0; sub < KSUB; sub++) {
-          mul[sub] = 8.0f * sc[nt * KSUB + sub];
+        for (int sub = 0; sub < SUBS; sub++) {
+          mul[sub] = 8.0f * sc[nt * SUBS + sub];
           c[sub] = __builtin_fmaf(-kBiasF, mul[sub], k0);
         }
         float t8[16];
 #pragma unroll
-        for (int r = 0; r < 16; r++) t8[r] = __builtin_fmaf(as_f(acc[nt][r]), mul[KSUB == 2 ? r / 8 : 0], c[KSUB == 2 ? r / 8 : 0]);
+        for (int r = 0; r < 16; r++) t8[r] = __builtin_fmaf(as_f(acc[nt][r]), mul[subof(r)], c[subof(r)]);
 #pragma unroll
         for (int q4 = 0; q4 < 4; q4++) {
           // all four bytes get written, so the 'old' operand of the first insertion is a don't-care
@@ -618,16 +641,16 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
     } else if constexpr (PV == 1) {
 #pragma unroll
       for (int nt = 0; nt < NT; nt++) {
-        float c[KSUB], mul[KSUB];
+        float c[SUBS], mul[SUBS];
 #pragma unroll
-        for (int sub = 0; sub < KSUB; sub++) {
-          c[sub] = MASK ? PSHIFT - m_used : __builtin_fmaf(-kBiasF, sc[nt * KSUB + sub], PSHIFT - m_used);
-          mul[sub] = MASK ? 1.0f : sc[nt * KSUB + sub];   // masked variants already hold scores
+        for (int sub = 0; sub < SUBS; sub++) {
+          c[sub] = MASK ? PSHIFT - m_used : __builtin_fmaf(-kBiasF, sc[nt * SUBS + sub], PSHIFT - m_used);
+          mul[sub] = MASK ? 1.0f : sc[nt * SUBS + sub];   // masked variants already hold scores
         }
         float p[16];
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-          p[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(as_f(acc[nt][r]), mul[KSUB == 2 ? r / 8 : 0], c[KSUB == 2 ? r / 8 : 0]));
+          p[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(as_f(acc[nt][r]), mul[subof(r)], c[subof(r)]));
           if constexpr (!MSUM) lsum += p[r];   // the unrounded sum, for LSE only
         }
 #pragma unroll
@@ -642,19 +665,19 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
     } else {
 #pragma unroll
       for (int nt = 0; nt < NT; nt++) {
-        float c[KSUB], mul[KSUB];
+        float c[SUBS], mul[SUBS];
 #pragma unroll
-        for (int sub = 0; sub < KSUB; sub++) {
-          c[sub] = MASK ? PSHIFT - m_used : __builtin_fmaf(-kBiasF, sc[nt * KSUB + sub], PSHIFT - m_used);
-          mul[sub] = MASK ? 1.0f : sc[nt * KSUB + sub];
+        for (int sub = 0; sub < SUBS; sub++) {
+          c[sub] = MASK ? PSHIFT - m_used : __builtin_fmaf(-kBiasF, sc[nt * SUBS + sub], PSHIFT - m_used);
+          mul[sub] = MASK ? 1.0f : sc[nt * SUBS + sub];
         }
         // fp16 probabilities are packed in place: registers 0-7 of each accumulator take the 16 halves
         // (v_cvt_pk_f16_f32, round to nearest even) once the two scores they replace have been consumed.
 #pragma unroll
         for (int r = 0; r < 16; r += 2) {
           v2f pp;
-          pp[0] = __builtin_amdgcn_exp2f(__builtin_fmaf(as_f(acc[nt][r]), mul[KSUB == 2 ? r / 8 : 0], c[KSUB == 2 ? r / 8 : 0]));
-          pp[1] = __builtin_amdgcn_exp2f(__builtin_fmaf(as_f(acc[nt][r + 1]), mul[KSUB == 2 ? r / 8 : 0], c[KSUB == 2 ? r / 8 : 0]));
+          pp[0] = __builtin_amdgcn_exp2f(__builtin_fmaf(as_f(acc[nt][r]), mul[subof(r)], c[subof(r)]));
+          pp[1] = __builtin_amdgcn_exp2f(__builtin_fmaf(as_f(acc[nt][r + 1]), mul[subof(r)], c[subof(r)]));
           lsum += pp[0];
           lsum += pp[1];
           acc[nt][r >> 1] = __builtin_bit_cast(int, __builtin_convertvector(pp, v2h));

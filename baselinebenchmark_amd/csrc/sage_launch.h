@@ -12,7 +12,7 @@ struct QuantArgs {
   int B, H, L, D;
   int64_t x_sb, x_sh, x_sn, o_sb, o_sh, o_sn, km_sb, km_sh;
   int blk;
-  int groups;   // scales per block: 1, or 8 (scale g covers the rows r of the block with r % 8 == g); fixed-length only
+  int groups;   // scales per block: 1; 8 (scale g covers the rows r of the block with r % 8 == g); 4 ((r % 8) / 2 == g); fixed-length only
   float mult;
   const int32_t* cu_seqlens;
   const int32_t* cu_blocks;
@@ -60,6 +60,7 @@ struct AttnArgs {
   int blkq, blkk;            // scale block sizes: powers of two (32, 64, 128)
   int blkq_shift, blkk_shift;  // their log2
   int qg_shift;              // log2 of the Q scales per block: 0, or 3 (eight interleaved scales: rows r, r + 8, ... share one)
+  int k_interleave;          // 1: four interleaved K scales per block (scale t for the keys n with (n % 8) / 2 == t); host-side dispatch only
   int out_bf16;
   int nqt;  // q-tiles per sequence (fixed-length mode)
   // packed mode (cu_q != nullptr)
@@ -98,6 +99,7 @@ hipError_t launch_attn(const AttnArgs& a, int D, int pv, bool causal, int grid, 
 hipError_t launch_attn_masked(const AttnArgs& a, int D, int pv, int grid, hipStream_t st);
 hipError_t launch_attn_qfused(const AttnArgs& a, int D, int pv, bool causal, int grid, hipStream_t st);
 hipError_t launch_attn_k16(const AttnArgs& a, int D, int pv, bool causal, int grid, hipStream_t st);
+hipError_t launch_attn_kinterleaved(const AttnArgs& a, int D, int pv, bool causal, int grid, hipStream_t st);
 hipError_t launch_varlen_plan(const int32_t* cu_q, const int32_t* cu_k, int nseq, int total_q, int blkq, int blkk, int bm,
                               int bn, int causal, int32_t* plan, hipStream_t st);
 

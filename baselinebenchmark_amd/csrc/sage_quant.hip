@@ -112,21 +112,23 @@ __global__ void __launch_bounds__(256) quant_int8_kernel(QuantArgs a) {
     __syncthreads();
     amax = fmaxf(fmaxf(wmax[0], wmax[1]), fmaxf(wmax[2], wmax[3]));
   } else {
-    // Eight interleaved scales per block: every row this lane holds has the same index modulo 8 (the passes are
-    // RPP rows apart, a multiple of 8), so the lane belongs to one group.  Maximum over the lanes of a row, then over
-    // the rows of the group through LDS (the values are non-negative floats: their bit patterns order like integers).
+    // Interleaved scales per block (eight: group = row % 8; four: group = (row % 8) / 2): every row this lane holds has
+    // the same index modulo 8 (the passes are RPP rows apart, a multiple of 8), so the lane belongs to one group.
+    // Maximum over the lanes of a row, then over the rows of the group through LDS (the values are non-negative
+    // floats: their bit patterns order like integers).
     static_assert(RPP % 8 == 0, "a lane's rows must share their index modulo 8");
     if (tid < 8) gmax[tid] = 0;
     __syncthreads();
 #pragma unroll
     for (int o = 1; o < TPR; o <<= 1) amax = fmaxf(amax, __shfl_xor(amax, o));
-    if (tc == 0) atomicMax(&gmax[tr & 7], __builtin_bit_cast(int, amax));
+    const int gid = a.groups == 8 ? (tr & 7) : ((tr & 7) >> 1);
+    if (tc == 0) atomicMax(&gmax[gid], __builtin_bit_cast(int, amax));
     __syncthreads();
-    amax = __builtin_bit_cast(float, gmax[tr & 7]);
+    amax = __builtin_bit_cast(float, gmax[gid]);
   }
   const float scale = fmaxf(amax / 127.0f, kScaleFloor);
   if (a.groups == 1) { if (tid == 0) a.scale[sidx] = scale; }
-  else if (tc == 0 && tr < 8) a.scale[sidx + tr] = scale;
+  else if (tc == 0 && tr < a.groups) a.scale[sidx + tr] = fmaxf(__builtin_bit_cast(float, gmax[tr]) / 127.0f, kScaleFloor);   // group tr's scale
 
   const float rcp = 1.0f / scale;
   // The fast correction-step division needs: significand of scale not all ones, and scale and rcp

@@ -99,12 +99,21 @@ def k_mean(k: torch.Tensor, tensor_layout: str = "HND") -> torch.Tensor:
 
 
 BLK_INTERLEAVE8 = 0x100   # SAGE_BLK_INTERLEAVE8 of the C ABI: eight interleaved scales per Q block
+BLK_INTERLEAVE4 = 0x200   # SAGE_BLK_INTERLEAVE4: four interleaved scales per K block
 
 
 def _check_interleave(q_interleave) -> int:
     if q_interleave not in (1, 8):
         raise ValueError("q_interleave must be 1 (one scale per Q block) or 8 (rows r, r+8, ... of a block share a scale)")
     return BLK_INTERLEAVE8 if q_interleave == 8 else 0
+
+
+def _check_k_interleave(k_interleave, BLKK) -> int:
+    if k_interleave not in (1, 4):
+        raise ValueError("k_interleave must be 1 (one scale per K block) or 4 (keys n with equal (n % 8) // 2 share a scale)")
+    if k_interleave == 4 and BLKK == 16:
+        raise NotImplementedError("four interleaved K scales need K blocks of 32, 64 or 128 keys")
+    return BLK_INTERLEAVE4 if k_interleave == 4 else 0
 
 
 def _quant_one(x, km, blk, mult, tensor_layout, groups=1):
@@ -121,19 +130,23 @@ def _quant_one(x, km, blk, mult, tensor_layout, groups=1):
             km = km.contiguous()
         km_sb, km_sh = (km.stride(0), km.stride(1)) if tensor_layout == "HND" else (km.stride(0), km.stride(2))
     check(lib().sage_quant_int8(_ptr(x), _ptr(out), _ptr(scale), _ptr(km), B, H, L, D, sb, sh, sn, osb, osh, osn,
-                                km_sb, km_sh, blk | _check_interleave(groups), mult, _dt(x.dtype), None, None, 0, _stream(x)))
+                                km_sb, km_sh, blk | {1: 0, 8: BLK_INTERLEAVE8, 4: BLK_INTERLEAVE4}[groups], mult, _dt(x.dtype),
+                                None, None, 0, _stream(x)))
     return out, scale
 
 
 @torch.no_grad()
-def per_block_int8(q, k, km=None, BLKQ=128, BLKK=64, sm_scale=None, tensor_layout="HND", q_interleave=1):
+def per_block_int8(q, k, km=None, BLKQ=128, BLKK=64, sm_scale=None, tensor_layout="HND", q_interleave=1, k_interleave=1):
     """Per-block INT8 quantisation of Q and K; returns (q_int8, q_scale, k_int8, k_scale).
 
     Same contract as quant_per_block.py:49-101: optional ``k - km`` in the input dtype, Q scaled by
     ``sm_scale * 1.44269504`` (default sm_scale = head_dim**-0.5), K by 1, scales [B, H, ceil(L/BLK)].
     ``q_interleave=8`` (no counterpart in the reference's code; the granularity upstream SageAttention calls per-thread,
     with WARPQ = BLKQ): every Q block gets eight scales, scale g for its rows r with r % 8 == g, and q_scale is
-    [B, H, ceil(L/BLKQ) * 8]; pass the same keyword to ``forward``.
+    [B, H, ceil(L/BLKQ) * 8]; pass the same keyword to ``forward``.  ``k_interleave=4`` is upstream's per-thread K
+    granularity (WARPK = BLKK): four scales per K block, scale t for its keys n with (n % 8) // 2 == t, k_scale
+    [B, H, ceil(L/BLKK) * 4].  ``per_block_int8(..., BLKQ=32, BLKK=64, q_interleave=8, k_interleave=4)`` is upstream's
+    per_thread_int8 with this reference's quantiser arithmetic.
     """
     _check_float("q", q)
     _check_float("k", k)
@@ -147,8 +160,9 @@ def per_block_int8(q, k, km=None, BLKQ=128, BLKK=64, sm_scale=None, tensor_layou
         raise ValueError("q and k head dimensions differ")
     _check_blocks_quant(BLKQ, BLKK)
     _check_interleave(q_interleave)
+    _check_k_interleave(k_interleave, BLKK)
     q_int8, q_scale = _quant_one(q, None, BLKQ, _q_mult(q.shape[-1], sm_scale), tensor_layout, q_interleave)
-    k_int8, k_scale = _quant_one(k, km, BLKK, 1.0, tensor_layout)
+    k_int8, k_scale = _quant_one(k, km, BLKK, 1.0, tensor_layout, k_interleave)
     return q_int8, q_scale, k_int8, k_scale
 
 
@@ -212,7 +226,7 @@ def _mask_args(attn_mask, B, Hq, Sq, Skv, device):
 @torch.no_grad()
 def forward(q, k, v, q_scale, k_scale, tensor_layout="HND", attn_mask=None, output_dtype=torch.float16,
             return_lse=False, maxnreg=None, block_m=None, num_warps=None, num_stages=None, backend=None,
-            BLKQ=128, BLKK=64, is_causal=False, pv_mode="fp16", q_interleave=1):
+            BLKQ=128, BLKK=64, is_causal=False, pv_mode="fp16", q_interleave=1, k_interleave=1):
     """Fused INT8-QK attention on operands produced by per_block_int8; returns (out, lse).
 
     Signature of sageattention_hip.py:55-56 / attn_qk_int8_per_block_native.py:438-453; the tuning
@@ -222,9 +236,13 @@ def forward(q, k, v, q_scale, k_scale, tensor_layout="HND", attn_mask=None, outp
     ``attn_mask``: boolean (True keeps the key) or additive bias on the base-2 logits, broadcastable
     to [B, Hq, Sq, Skv] (sageattention_triton.py:92-105); not combinable with ``is_causal``.
     ``lse`` is base 2 (sageattention_triton.py:127-129) and an empty tensor unless requested.
-    ``q_interleave=8``: q_scale holds eight interleaved scales per Q block (see per_block_int8).
+    ``q_interleave=8`` / ``k_interleave=4``: q_scale / k_scale hold eight / four interleaved scales per block (see
+    per_block_int8); interleaved K scales cannot be combined with ``attn_mask``.
     """
     qflag = _check_interleave(q_interleave)
+    kflag = _check_k_interleave(k_interleave, BLKK)
+    if kflag and attn_mask is not None:
+        raise NotImplementedError("interleaved K scales cannot be combined with attn_mask")
     for name, t in (("q", q), ("k", k)):
         if not isinstance(t, torch.Tensor) or not t.is_cuda or t.dtype != torch.int8 or not t.is_contiguous():
             raise TypeError(f"{name} must be contiguous GPU INT8")
@@ -251,7 +269,7 @@ def forward(q, k, v, q_scale, k_scale, tensor_layout="HND", attn_mask=None, outp
     if BLKQ not in (16, 32, 64, 128) or BLKK not in (16, 32, 64, 128):
         raise NotImplementedError("the attention kernel needs Q and K scale blocks of 16, 32, 64 or 128 rows")
     exp_q = (B, Hq, (Sq + BLKQ - 1) // BLKQ * q_interleave)
-    exp_k = (B, Hkv, (Skv + BLKK - 1) // BLKK)
+    exp_k = (B, Hkv, (Skv + BLKK - 1) // BLKK * k_interleave)
     if tuple(q_scale.shape) != exp_q:
         raise ValueError(f"q_scale has shape {tuple(q_scale.shape)}, expected {exp_q}")
     if tuple(k_scale.shape) != exp_k:
@@ -276,17 +294,19 @@ def forward(q, k, v, q_scale, k_scale, tensor_layout="HND", attn_mask=None, outp
     check(lib().sage_attn_fwd(_ptr(q), _ptr(k), _ptr(panels), _ptr(q_scale.contiguous()), _ptr(k_scale.contiguous()),
                               _ptr(v_scale), _ptr(out), _ptr(lse if return_lse else None),
                               B, Hq, Hkv, Sq, Skv, D, qsb, qsh, qsn, ksb, ksh, ksn, osb, osh, osn,
-                              BLKQ | qflag, BLKK, int(bool(is_causal)), pv, _dt(output_dtype),
+                              BLKQ | qflag, BLKK | kflag, int(bool(is_causal)), pv, _dt(output_dtype),
                               None, None, None, 0, 0, 0, 0, _stream(q)))
     return out, lse
 
 
 @torch.no_grad()
 def forward_fused_q(q, k, v, k_scale, tensor_layout="HND", sm_scale=None, output_dtype=None, return_lse=False,
-                    BLKQ=128, BLKK=64, is_causal=False, pv_mode="fp16"):
+                    BLKQ=128, BLKK=64, is_causal=False, pv_mode="fp16", k_interleave=1):
     """forward() for a floating-point ``q`` and an already quantised ``k``: each q-tile is quantised inside the
     attention kernel (bit-identical to per_block_int8 on q followed by forward()).  For callers that keep K
-    quantised across calls.  ``k``/``k_scale`` as returned by per_block_int8; returns (out, lse) like forward()."""
+    quantised across calls.  ``k``/``k_scale`` as returned by per_block_int8 (``k_interleave=4``: with four interleaved
+    scales per K block); returns (out, lse) like forward()."""
+    kflag = _check_k_interleave(k_interleave, BLKK)
     _check_float("q", q)
     _check_float("v", v)
     if not isinstance(k, torch.Tensor) or not k.is_cuda or k.dtype != torch.int8 or not k.is_contiguous():
@@ -307,8 +327,8 @@ def forward_fused_q(q, k, v, k_scale, tensor_layout="HND", sm_scale=None, output
         raise NotImplementedError("head_dim must be 64 or 128")
     if BLKQ not in (16, 32, 64, 128) or BLKK not in (16, 32, 64, 128):
         raise NotImplementedError("the fused-Q kernel needs Q and K scale blocks of 16, 32, 64 or 128 rows")
-    if tuple(k_scale.shape) != (B, Hkv, (Skv + BLKK - 1) // BLKK):
-        raise ValueError(f"k_scale has shape {tuple(k_scale.shape)}, expected {(B, Hkv, (Skv + BLKK - 1) // BLKK)}")
+    if tuple(k_scale.shape) != (B, Hkv, (Skv + BLKK - 1) // BLKK * k_interleave):
+        raise ValueError(f"k_scale has shape {tuple(k_scale.shape)}, expected {(B, Hkv, (Skv + BLKK - 1) // BLKK * k_interleave)}")
     pv = _pv(pv_mode)
     panels, v_scale = prepare_v(v, tensor_layout, pv)
     out = torch.empty(q.shape, device=q.device, dtype=output_dtype)
@@ -318,7 +338,7 @@ def forward_fused_q(q, k, v, k_scale, tensor_layout="HND", sm_scale=None, output
                                      _ptr(panels), _ptr(k_scale.contiguous()), _ptr(v_scale), _ptr(out),
                                      _ptr(lse if return_lse else None),
                                      B, Hq, Hkv, Sq, Skv, D, qsb, qsh, qsn, ksb, ksh, ksn, osb, osh, osn,
-                                     BLKQ, BLKK, int(bool(is_causal)), pv, _dt(output_dtype), None, None, None, 0, 0, 0,
+                                     BLKQ, BLKK | kflag, int(bool(is_causal)), pv, _dt(output_dtype), None, None, None, 0, 0, 0,
                                      _stream(q)))
     return out, lse
 
@@ -346,7 +366,8 @@ def _apply_recipe(quant_recipe, BLKQ, BLKK, pv_mode):
 @torch.no_grad()
 def sageattn(q, k, v, tensor_layout="HND", is_causal=False, sm_scale=None, smooth_k=True, pv_mode=None,
              BLKQ=128, BLKK=64, return_lse=False, qk_quant_dtype="int8", quant_recipe=None, attn_mask=None,
-             cu_seqlens_q=None, cu_seqlens_k=None, max_seqlen_q=None, max_seqlen_k=None, q_interleave=1, **kwargs):
+             cu_seqlens_q=None, cu_seqlens_k=None, max_seqlen_q=None, max_seqlen_k=None, q_interleave=1,
+             k_interleave=1, **kwargs):
     """Quantise + attend in one call: out = softmax(q k^T * sm_scale [causal | + attn_mask]) v.
 
     Returns ``out`` (q's shape and dtype), or ``(out, lse)`` with ``return_lse=True`` where lse is
@@ -361,7 +382,8 @@ def sageattn(q, k, v, tensor_layout="HND", is_causal=False, sm_scale=None, smoot
     q is then [total_q, Hq, D], k and v [total_k, Hkv, D], ``tensor_layout`` is not consulted, ``max_seqlen_q`` /
     ``max_seqlen_k`` bound the sequence lengths (derived from cu_seqlens, with one host synchronisation, when left
     out), and lse comes back as [Hq, total_q]; see sageattn_varlen, which this call is then identical to.
-    ``q_interleave=8``: eight interleaved Q scales per block (see per_block_int8); fixed-length batches only.
+    ``q_interleave=8`` / ``k_interleave=4``: eight interleaved Q scales / four interleaved K scales per block (see
+    per_block_int8); fixed-length batches only, and interleaved K scales not together with ``attn_mask``.
     """
     if qk_quant_dtype != "int8":
         raise NotImplementedError("only INT8 Q/K quantisation is implemented")
@@ -369,9 +391,12 @@ def sageattn(q, k, v, tensor_layout="HND", is_causal=False, sm_scale=None, smoot
         raise TypeError(f"unexpected arguments: {sorted(kwargs)}")
     BLKQ, BLKK, pv_mode = _apply_recipe(quant_recipe, BLKQ, BLKK, pv_mode)
     qflag = _check_interleave(q_interleave)
+    kflag = _check_k_interleave(k_interleave, BLKK)
+    if kflag and attn_mask is not None:
+        raise NotImplementedError("interleaved K scales cannot be combined with attn_mask")
     if cu_seqlens_q is not None or cu_seqlens_k is not None:
-        if qflag:
-            raise NotImplementedError("interleaved Q scales are not supported for packed batches")
+        if qflag or kflag:
+            raise NotImplementedError("interleaved scales are not supported for packed batches")
         if attn_mask is not None:
             raise NotImplementedError("attn_mask is not supported for packed batches")
         cu_seqlens_k = cu_seqlens_q if cu_seqlens_k is None else cu_seqlens_k
@@ -406,7 +431,7 @@ def sageattn(q, k, v, tensor_layout="HND", is_causal=False, sm_scale=None, smoot
     out = torch.empty(q.shape, device=q.device, dtype=q.dtype)
     _, _, _, _, osb, osh, osn = _layout(out, tensor_layout)
     lse = torch.empty((B, Hq, Sq), device=q.device, dtype=torch.float32) if return_lse else None
-    ws_bytes = lib().sage_sageattn_workspace_bytes(B, Hq, Hkv, Sq, Skv, D, BLKQ | qflag, BLKK, pv, 0, 0, 0)
+    ws_bytes = lib().sage_sageattn_workspace_bytes(B, Hq, Hkv, Sq, Skv, D, BLKQ | qflag, BLKK | kflag, pv, 0, 0, 0)
     ws = torch.empty(max(ws_bytes, 256), device=q.device, dtype=torch.uint8)
     if attn_mask is not None:
         if is_causal:
@@ -420,7 +445,7 @@ def sageattn(q, k, v, tensor_layout="HND", is_causal=False, sm_scale=None, smoot
     else:
         check(lib().sage_sageattn(_ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _ptr(ws), ws_bytes,
                                   B, Hq, Hkv, Sq, Skv, D, qsb, qsh, qsn, ksb, ksh, ksn, vsb, vsh, vsn, osb, osh, osn,
-                                  _dt(q.dtype), BLKQ | qflag, BLKK, float(D ** -0.5 if sm_scale is None else sm_scale),
+                                  _dt(q.dtype), BLKQ | qflag, BLKK | kflag, float(D ** -0.5 if sm_scale is None else sm_scale),
                                   int(bool(is_causal)), int(bool(smooth_k)), pv, None, None, 0, 0, _stream(q)))
     if return_lse:
         return out, lse * 0.6931471805599453

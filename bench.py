@@ -29,7 +29,8 @@ PEAK_FP16 = 2516.6       # dense FP16 MFMA peak, TFLOP/s
 
 
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "attn_kernel_traffic.json")
-KERNEL_SOURCES = ["sage_attn_kernel.h", "sage_attn.hip", "sage_attn_qfuse.hip", "sage_attn_mask.hip", "sage_common.h", "sage_launch.h"]
+KERNEL_SOURCES = ["sage_attn_kernel.h", "sage_attn.hip", "sage_attn_qfuse.hip", "sage_attn_mask.hip", "sage_attn_kinterleave.hip",
+                  "sage_common.h", "sage_launch.h"]
 
 
 def kernel_source_digest() -> str:

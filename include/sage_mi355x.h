@@ -53,6 +53,13 @@ extern "C" {
  * quant_per_block.py:38-46 applied per row group.  Fixed-length batches only; not for K; the Q quantisation fused into the
  * attention kernel (sage_attn_fwd_qfused) does not take it -- sage_sageattn* run the standalone Q pass instead. */
 #define SAGE_BLK_INTERLEAVE8 0x100
+/* The same for K (upstream's per-thread K granularity, its WARPK = blkk): OR-ed into `blk` of sage_quant_int8 when it
+ * quantises K and into `blkk` of sage_attn_fwd, sage_attn_fwd_qfused, sage_sageattn* and sage_sageattn_workspace_bytes,
+ * every block of blkk = 32, 64 or 128 keys carries FOUR scales, scale t for the keys n of the block with (n % 8) / 2 == t
+ * (keys 2t, 2t+1, 2t+8, 2t+9, ...): scale[(b*H + h)*ceil(S/blkk)*4 + block*4 + t].  In the transposed score tile a lane
+ * holds keys of exactly two of the four groups per 32 keys, so the kernel applies two scales per lane and 32-key group.
+ * Fixed-length batches only; not with an explicit mask. */
+#define SAGE_BLK_INTERLEAVE4 0x200
 
 /* Rows of K/V covered by one V panel (see sage_prep_v). */
 #define SAGE_PANEL_ROWS 128
@@ -78,8 +85,8 @@ const char* sage_last_error(void);
  * scale:  fp32; fixed-length: scale[(b*H + h)*ceil(L/blk) + block];
  *         packed: scale[h*scale_sh + cu_blocks[b] + block] (cu_blocks from sage_varlen_plan).
  * mult:   sm_scale*1.44269504 for Q (quant_per_block.py:87), 1.0 for K (:97).
- * blk in {16,32,64,128}, optionally | SAGE_BLK_INTERLEAVE8 (Q only, fixed-length only); D in {64,128}.  In packed mode L
- * is the longest sequence.
+ * blk in {16,32,64,128}, optionally | SAGE_BLK_INTERLEAVE8 or, for 32 rows and more, | SAGE_BLK_INTERLEAVE4 (fixed-length
+ * only); D in {64,128}.  In packed mode L is the longest sequence.
  */
 int sage_quant_int8(const void* x, int8_t* out, float* scale, const void* km,
                     int B, int H, int L, int D,

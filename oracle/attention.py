@@ -34,13 +34,15 @@ def expand_scale(scale: torch.Tensor, block: int, length: int) -> torch.Tensor:
 
 
 def expand_scale_interleaved(scale: torch.Tensor, block: int, groups: int, length: int) -> torch.Tensor:
-    """Row n takes scale[(n // block) * groups + n % groups]: ``groups`` interleaved scales per block."""
+    """Interleaved scales per block: eight -> row n takes scale[(n // block) * 8 + n % 8]; four -> scale[(n // block) * 4 +
+    (n % 8) // 2]."""
     n = torch.arange(length)
-    return scale[..., (n // block) * groups + n % groups, None]
+    g = n % 8 if groups == 8 else (n % 8) // 2
+    return scale[..., (n // block) * groups + g, None]
 
 
 def sage_reference(q_int8, k_int8, v, q_scale, k_scale, tensor_layout="HND", BLKQ=128, BLKK=64,
-                   is_causal=False, attn_mask=None, v_scale=None, dtype=torch.float64, q_interleave=1):
+                   is_causal=False, attn_mask=None, v_scale=None, dtype=torch.float64, q_interleave=1, k_interleave=1):
     """Attention on already-quantised operands.  Returns (out [layout of q], lse2 [B,Hq,Sq]).
 
     * v may be fp16/bf16/fp32, or float8_e4m3fn together with ``v_scale`` [B,Hkv,D]
@@ -48,7 +50,8 @@ def sage_reference(q_int8, k_int8, v, q_scale, k_scale, tensor_layout="HND", BLK
     * causal mask is top-left aligned (key j visible to query i iff j <= i), which is
       torch SDPA's ``is_causal=True`` convention.
     * rows with no visible key give out = 0 and lse = -inf.
-    * ``q_interleave`` = 8: q_scale holds eight interleaved scales per Q block (oracle.quant.quant_per_block_int8).
+    * ``q_interleave`` = 8 / ``k_interleave`` = 4: q_scale / k_scale hold eight / four interleaved scales per block
+      (oracle.quant.quant_per_block_int8).
     """
     q = _hnd(q_int8, tensor_layout).cpu().to(dtype)
     k = _hnd(k_int8, tensor_layout).cpu().to(dtype)
@@ -58,7 +61,8 @@ def sage_reference(q_int8, k_int8, v, q_scale, k_scale, tensor_layout="HND", BLK
     sq, skv = q.shape[-2], k.shape[-2]
     q = q * (expand_scale(q_scale.cpu().to(dtype), BLKQ, sq) if q_interleave == 1 else
              expand_scale_interleaved(q_scale.cpu().to(dtype), BLKQ, q_interleave, sq))
-    k = k * expand_scale(k_scale.cpu().to(dtype), BLKK, skv)
+    k = k * (expand_scale(k_scale.cpu().to(dtype), BLKK, skv) if k_interleave == 1 else
+             expand_scale_interleaved(k_scale.cpu().to(dtype), BLKK, k_interleave, skv))
     group = q.shape[1] // k.shape[1]
     k = k.repeat_interleave(group, dim=1)
     vv = vv.repeat_interleave(group, dim=1)

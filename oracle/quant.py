@@ -9,7 +9,7 @@ Reference lines followed:
   * host     backends/_enflame/ops/sage_attention/quant_per_block.py:49-101
   * guard    backends/_hygon/ops/sageattention/sageattention_triton.py:35
 Parity unpinned (not in the reference's code, defined here and pinned against the mathematics in the tests): k_mean,
-quant_v_fp8, and the eight interleaved scales per block of quant_per_block_int8(groups=8).
+quant_v_fp8, and the interleaved scales per block of quant_per_block_int8(groups=8 or 4).
 """
 from __future__ import annotations
 
@@ -53,10 +53,11 @@ def quant_per_block_int8(x_hnd32: np.ndarray, blk: int, mult, groups: int = 1) -
 
     Vectorised over tiles; identical arithmetic to ``quant_tile_int8``.
     Grid of quant_per_block.py:81 / :91: one program per (block, head, batch).
-    ``groups`` = 8: eight interleaved scales per block, scale g for the rows r of the block with r % 8 == g (the
-    granularity upstream SageAttention calls per-thread, with its WARPQ = blk).  The reference has no code for it
-    (parity unpinned): it is defined here as the same tile arithmetic applied to each row group, and pinned in the
-    tests against a row-by-row loop over ``quant_tile_int8``.
+    ``groups`` = 8: eight interleaved scales per block, scale g for the rows r of the block with r % 8 == g;
+    ``groups`` = 4: four, scale t for the rows with (r % 8) // 2 == t (the granularities upstream SageAttention calls
+    per-thread for Q and K, with its WARPQ / WARPK = blk).  The reference has no code for them (parity unpinned): they
+    are defined here as the same tile arithmetic applied to each row group, and pinned in the tests against a
+    row-group loop over ``quant_tile_int8``.
     """
     B, H, L, C = x_hnd32.shape
     nblk = (L + blk - 1) // blk
@@ -64,11 +65,12 @@ def quant_per_block_int8(x_hnd32: np.ndarray, blk: int, mult, groups: int = 1) -
     x = x_hnd32.astype(np.float32, copy=False) * np.float32(mult)
     if pad:
         x = np.concatenate([x, np.zeros((B, H, pad, C), np.float32)], axis=2)
-    # [.., block, row group member, group, channel]: with groups == 1 a block is one group of blk rows
-    xt = x.reshape(B, H, nblk, blk // groups, groups, C)
-    amax = np.max(np.abs(xt), axis=(3, 5)).astype(np.float32)
+    # [.., block, octet of rows, group, rows of the group inside the octet, channel]; one group: the whole block
+    per_octet = {1: 1, 8: 1, 4: 2}[groups]
+    xt = x.reshape(B, H, nblk, blk // (groups * per_octet), groups, per_octet, C)
+    amax = np.max(np.abs(xt), axis=(3, 5, 6)).astype(np.float32)
     scale = np.maximum(amax / np.float32(127.0), SCALE_FLOOR).astype(np.float32)          # [B, H, nblk, groups]
-    z = xt / scale[:, :, :, None, :, None]
+    z = xt / scale[:, :, :, None, :, None, None]
     z = z + np.float32(0.5) * np.where(z >= 0, np.float32(1.0), np.float32(-1.0)).astype(np.float32)
     q = np.trunc(z).astype(np.int32).astype(np.int8).reshape(B, H, nblk * blk, C)[:, :, :L]
     return np.ascontiguousarray(q), np.ascontiguousarray(scale.reshape(B, H, nblk * groups))
@@ -90,12 +92,12 @@ def q_multiplier(head_dim: int, sm_scale=None) -> np.float32:
     return np.float32(float(sm_scale) * LOG2E_REF)
 
 
-def per_block_int8(q, k, km=None, BLKQ=128, BLKK=64, sm_scale=None, tensor_layout="HND", q_interleave=1):
+def per_block_int8(q, k, km=None, BLKQ=128, BLKK=64, sm_scale=None, tensor_layout="HND", q_interleave=1, k_interleave=1):
     """Restates per_block_int8 (quant_per_block.py:49-101) on CPU tensors.
 
     Returns torch CPU tensors (q_int8, q_scale, k_int8, k_scale) with the reference's
     shapes: int8 like q / k, scales [B, H, ceil(L/BLK)] float32 (q_scale [B, H, ceil(L/BLKQ)*8] with
-    ``q_interleave=8``, see quant_per_block_int8).
+    ``q_interleave=8``, k_scale [B, H, ceil(L/BLKK)*4] with ``k_interleave=4``, see quant_per_block_int8).
     """
     if km is not None:
         k = k - km  # input-dtype subtraction, quant_per_block.py:53-54
@@ -103,7 +105,7 @@ def per_block_int8(q, k, km=None, BLKQ=128, BLKK=64, sm_scale=None, tensor_layou
     k32 = _hnd(_to_f32(k), tensor_layout)
     head_dim = q32.shape[-1]
     qi, qs = quant_per_block_int8(q32, BLKQ, q_multiplier(head_dim, sm_scale), q_interleave)
-    ki, ks = quant_per_block_int8(k32, BLKK, np.float32(1.0))
+    ki, ks = quant_per_block_int8(k32, BLKK, np.float32(1.0), k_interleave)
     qi = np.ascontiguousarray(_hnd(qi, tensor_layout)) if tensor_layout == "NHD" else qi
     ki = np.ascontiguousarray(_hnd(ki, tensor_layout)) if tensor_layout == "NHD" else ki
     return (torch.from_numpy(qi), torch.from_numpy(qs), torch.from_numpy(ki), torch.from_numpy(ks))

@@ -43,6 +43,8 @@ def test_size_queries_do_not_need_a_gpu(sage_lib):
     a = sage_lib.sage_sageattn_workspace_bytes(1, 4, 4, 4096, 4096, 128, 32, 64, 1, 0, 0, 0)
     b = sage_lib.sage_sageattn_workspace_bytes(1, 4, 4, 4096, 4096, 128, 32 | 0x100, 64, 1, 0, 0, 0)
     assert b - a == 4 * 128 * 7 * 4
+    c = sage_lib.sage_sageattn_workspace_bytes(1, 4, 4, 4096, 4096, 128, 32, 64 | 0x200, 1, 0, 0, 0)
+    assert c - a == 4 * 64 * 3 * 4                      # four interleaved K scales per block of 64 keys
     n = sage_lib.sage_varlen_plan_ints(16, 266000)
     offs = (ctypes.c_int64 * 5)()
     sage_lib.sage_varlen_plan_offsets(16, 266000, offs)
@@ -86,7 +88,9 @@ def test_attn_argument_errors(sage_lib):
     assert call(pv=1) == _cabi.SAGE_EINVAL           # fp8 needs v_scale
     assert call(pv=5) == _cabi.SAGE_EINVAL
     # interleaved Q scales (SAGE_BLK_INTERLEAVE8 = 0x100 OR-ed into blkq): a Q granularity of fixed-length batches
-    assert call(blkk=64 | 0x100) == _cabi.SAGE_ENOTIMPL
+    assert call(blkk=64 | 0x100) == _cabi.SAGE_ENOTIMPL      # eight scales per block are a Q granularity ...
+    assert call(blkq=64 | 0x200) == _cabi.SAGE_ENOTIMPL      # ... four a K granularity (SAGE_BLK_INTERLEAVE4 = 0x200)
+    assert call(blkk=16 | 0x200) == _cabi.SAGE_ENOTIMPL      # of blocks of 32 keys and more
     assert call(blkq=8 | 0x100) == _cabi.SAGE_ENOTIMPL
     rc = sage_lib.sage_attn_fwd(FAKE, FAKE, FAKE, FAKE, FAKE, NULL, FAKE, NULL, 1, 4, 2, 128, 128, 128,
                                 0, 128 * 128, 128, 0, 128 * 128, 128, 0, 128 * 128, 128, 32 | 0x100, 64, 0, 0, 0,

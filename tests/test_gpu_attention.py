@@ -326,6 +326,75 @@ def test_interleaved_q_scales(layout, pv, causal, blkq, D):
     assert torch.equal(one, two)
 
 
+@pytest.mark.parametrize("layout", ["HND", "NHD"])
+@pytest.mark.parametrize("pv", ["fp16", "fp8"])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("blkk,D,qi", [(64, 128, 8), (32, 128, 1), (128, 128, 8), (64, 64, 8), (128, 64, 1)])
+def test_interleaved_k_scales(layout, pv, causal, blkk, D, qi):
+    """Four interleaved K scales per block (keys n with equal (n % 8) // 2 share one; upstream's per-thread K granularity,
+    no code in the reference), alone and together with eight interleaved Q scales: `forward` against the reference
+    formula with the scales expanded key by key, with LSE; the kernels that quantise their own Q and the one-call
+    pipeline equal to the two steps bit for bit."""
+    g = torch.Generator().manual_seed(818 + blkk + D + int(causal) + qi)
+    B, Hq, Hkv, Sq, Skv = 2, 4, 2, 301, 301 if causal else 391
+    q = randn(layout, B, Hq, Sq, D, torch.bfloat16, g)
+    k = randn(layout, B, Hkv, Skv, D, torch.bfloat16, g)
+    v = randn(layout, B, Hkv, Skv, D, torch.bfloat16, g)
+    (k if layout == "HND" else k.transpose(1, 2))[1, 1, 130:132] *= 20.0    # two outlier keys: one scale group of one block
+    qd, kd, vd = q.to(DEV), k.to(DEV), v.to(DEV)
+    qi8, qs, ki, ks = sa.per_block_int8(qd, kd, BLKQ=32, BLKK=blkk, tensor_layout=layout, q_interleave=qi, k_interleave=4)
+    assert tuple(ks.shape) == (B, Hkv, (Skv + blkk - 1) // blkk * 4)
+    kw = dict(tensor_layout=layout, BLKQ=32, BLKK=blkk, is_causal=causal, pv_mode=pv, q_interleave=qi, k_interleave=4)
+    out, lse = sa.forward(qi8, ki, vd, qs, ks, return_lse=True, output_dtype=torch.bfloat16, **kw)
+    torch.cuda.synchronize()
+    ref, ref_lse = oa.sage_reference(qi8.cpu(), ki.cpu(), v, qs.cpu(), ks.cpu(), layout, 32, blkk, is_causal=causal,
+                                     q_interleave=qi, k_interleave=4)
+    m = oa.metrics(out.cpu().float(), ref)
+    assert m["finite"] and (m["rel_rmse"] < 6e-3 if pv == "fp16" else (m["cosine"] >= 0.999 and m["rel_rmse"] < 5e-2)), m
+    assert (lse.cpu().double() - ref_lse).abs().max().item() < (5e-3 if pv == "fp16" else 3e-2)
+    with pytest.raises(ValueError):      # a k_scale of the per-block shape is refused
+        sa.forward(qi8, ki, vd, qs, ks[..., ::4].contiguous(), **kw)
+    with pytest.raises(NotImplementedError):
+        sa.forward(qi8, ki, vd, qs, ks, attn_mask=torch.ones((1, 1, Sq, Skv), dtype=torch.bool, device=DEV),
+                   **{**kw, "is_causal": False})
+    plain, _ = sa.forward(qi8, ki, vd, qs, ks, output_dtype=torch.bfloat16, **kw)       # (no LSE: row sums on the matrix pipe)
+    if qi == 1:
+        fused, _ = sa.forward_fused_q(qd, ki, vd, ks, tensor_layout=layout, BLKQ=32, BLKK=blkk, is_causal=causal, pv_mode=pv,
+                                      k_interleave=4)
+        assert torch.equal(fused, plain)
+    one = sa.sageattn(qd, kd, vd, tensor_layout=layout, is_causal=causal, smooth_k=False, pv_mode=pv, BLKQ=32, BLKK=blkk,
+                      q_interleave=qi, k_interleave=4)
+    assert torch.equal(one, plain)
+
+
+def test_upstream_per_thread_granularity_against_fp32_sdpa():
+    """Q blocks of 32 rows with eight interleaved scales and K blocks of 64 keys with four (upstream's per_thread_int8:
+    WARPQ = 32, WARPK = 64), K smoothing, LSE: the one-call pipeline against FP32 SDPA on the raw inputs, and at least as
+    accurate as one scale per block."""
+    g = torch.Generator().manual_seed(919)
+    B, Hq, Hkv, S, D = 1, 8, 2, 1000, 128
+    q = randn("HND", B, Hq, S, D, torch.bfloat16, g)
+    k = randn("HND", B, Hkv, S, D, torch.bfloat16, g, offset_std=2.0)
+    v = randn("HND", B, Hkv, S, D, torch.bfloat16, g)
+    q[0, :, 5::37] *= 6.0
+    k[0, :, 3::41] *= 6.0
+    ref = oa.sdpa_fp32(q, k, v, "HND", True)
+    qd, kd, vd = q.to(DEV), k.to(DEV), v.to(DEV)
+    fine, lse = sa.sageattn(qd, kd, vd, is_causal=True, return_lse=True, BLKQ=32, BLKK=64, q_interleave=8, k_interleave=4)
+    coarse, lse_c = sa.sageattn(qd, kd, vd, is_causal=True, return_lse=True, BLKQ=32, BLKK=64)
+    mf, mc = oa.metrics(fine.cpu().float(), ref), oa.metrics(coarse.cpu().float(), ref)
+    assert mf["finite"] and mf["cosine"] >= 0.999 and mf["rmse"] <= mc["rmse"] * 1.02, (mf, mc)
+    # LSE of the original logits: the x6 outlier rows and keys make logits of +-40, whose INT8 error is what both
+    # granularities are measured by (the reference's bound for N(0,1) data is 1.5e-1, test_sage_attention_mate.py:171-178)
+    qq, kk = q.double(), k.double().repeat_interleave(4, 1)
+    logits = (qq @ kk.transpose(-1, -2) * D ** -0.5).masked_fill(torch.ones(S, S, dtype=torch.bool).triu(1), -float("inf"))
+    exact = torch.logsumexp(logits, -1)
+    ef, ec = (lse.cpu().double() - exact).abs(), (lse_c.cpu().double() - exact).abs()
+    # (measured: mean error 0.076 against 0.19 with one scale per block; the worst row, outlier query on outlier keys, 2.0)
+    assert torch.isfinite(ef).all() and ef.mean().item() <= 0.7 * ec.mean().item() and ef.mean().item() < 0.15, (ef.max(), ef.mean(), ec.mean())
+    assert ef.max().item() <= ec.max().item() * 1.05, (ef.max(), ec.max())
+
+
 def test_interleaved_q_scales_with_mask_lse_and_smoothing_against_fp32_sdpa():
     """sageattn(q_interleave=8) with K smoothing, LSE and an additive mask: against FP32 SDPA on the raw inputs."""
     g = torch.Generator().manual_seed(909)

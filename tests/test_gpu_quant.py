@@ -49,6 +49,35 @@ def test_interleaved_q_scales_bit_exact(layout, dtype, D, BLKQ):
         sa.per_block_int8(q.to(DEV), k.to(DEV), q_interleave=4)
 
 
+@pytest.mark.parametrize("layout", ["HND", "NHD"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("BLKK", [32, 64, 128])
+def test_interleaved_k_scales_bit_exact(layout, dtype, D, BLKK):
+    """Four interleaved scales per K block (keys n with equal (n % 8) // 2 share one), with K smoothing: int8 values
+    and scales equal the oracle's bit for bit; together with eight interleaved Q scales this is upstream's
+    per_thread_int8 granularity."""
+    g = torch.Generator().manual_seed(78 + D + BLKK)
+    q = randn(layout, 2, 3, 130, D, dtype, g)
+    k = randn(layout, 2, 3, 301, D, dtype, g, offset_std=2.0)
+    kv = k if layout == "HND" else k.transpose(1, 2)
+    kv[0, 1, 70:72] *= 30.0
+    kv[1, 2, 256:264] = kv[1, 2, 255:256]
+    km = oq.k_mean(k, layout)
+    out = sa.per_block_int8(q.to(DEV), k.to(DEV), km=km.to(DEV), BLKQ=32, BLKK=BLKK, tensor_layout=layout, q_interleave=8,
+                            k_interleave=4)
+    ref = oq.per_block_int8(q, k, km=km, BLKQ=32, BLKK=BLKK, tensor_layout=layout, q_interleave=8, k_interleave=4)
+    torch.cuda.synchronize()
+    assert tuple(out[3].shape) == (2, 3, (301 + BLKK - 1) // BLKK * 4)
+    for name, a, b in zip(("q_int8", "q_scale", "k_int8", "k_scale"), out, ref):
+        assert a.dtype == b.dtype and tuple(a.shape) == tuple(b.shape), name
+        assert torch.equal(a.cpu(), b), f"{name}: {(a.cpu() != b).sum().item()} mismatches"
+    with pytest.raises(ValueError):
+        sa.per_block_int8(q.to(DEV), k.to(DEV), k_interleave=8)
+    with pytest.raises(NotImplementedError):
+        sa.per_block_int8(q.to(DEV), k.to(DEV), BLKK=16, k_interleave=4)
+
+
 def test_reference_golden_vectors(golden):
     for name in golden["cases"]:
         c = golden_case(golden, str(name))

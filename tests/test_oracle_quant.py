@@ -227,3 +227,27 @@ def test_interleaved_q_scales_equal_the_tile_quantiser_applied_to_each_row_group
     _, s1 = oq.quant_per_block_int8(x, 32, 0.3)
     assert s8[0, 1, 8 + 1] == s1[0, 1, 1] and (s8[0, 1, 8:16] <= s1[0, 1, 1]).all() and s8[0, 1, 8] < 0.2 * s1[0, 1, 1]
 
+
+def test_four_interleaved_scales_equal_the_tile_quantiser_applied_to_each_key_group():
+    """Four interleaved scales per block (scale t for the rows r with (r % 8) // 2 == t: upstream's per-thread K
+    granularity; no code in the reference, parity unpinned): the vectorised oracle against the row-group loop."""
+    rng = np.random.default_rng(6)
+    x = rng.standard_normal((1, 2, 150, 64)).astype(np.float32)
+    x[0, 1, 70:72] *= np.float32(50.0)
+    for blk in (32, 64, 128):
+        q4, s4 = oq.quant_per_block_int8(x, blk, 1.0, 4)
+        nblk = (150 + blk - 1) // blk
+        assert s4.shape == (1, 2, nblk * 4)
+        for h in range(2):
+            for t in range(nblk):
+                for g in range(4):
+                    rows = [r for r in range(t * blk, min(150, (t + 1) * blk)) if (r % 8) // 2 == g]
+                    if not rows:
+                        assert s4[0, h, t * 4 + g] == oq.SCALE_FLOOR
+                        continue
+                    qq, ss = oq.quant_tile_int8(x[0, h, rows], 1.0)
+                    assert ss == s4[0, h, t * 4 + g] and np.array_equal(qq, q4[0, h, rows]), (blk, h, t, g)
+    _, s4 = oq.quant_per_block_int8(x, 64, 1.0, 4)
+    _, s1 = oq.quant_per_block_int8(x, 64, 1.0)
+    assert s4[0, 1, 4 + 3] == s1[0, 1, 1] and s4[0, 1, 4 + 0] < 0.2 * s1[0, 1, 1]      # rows 70, 71: group 3 of block 1
+
