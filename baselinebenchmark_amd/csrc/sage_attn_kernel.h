@@ -200,24 +200,40 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
     // rounds the balance of the last one matters more than locality -- 5 % on 4 x 32 heads of 4096 rows.)
     if ((U & 7) == 0 && (NG & 7) == 0 && (!CAUSAL || a.nqt * (U >> 3) >= 512)) {
       // Inside an XCD (workgroup index modulo 8; 32 compute units) the workgroups that run at the same time take
-      // neighbouring q-tiles of FEW heads: a tier is R consecutive q-tiles (by weight) of each of 32 / R heads.  Tiers go
-      // head group by head group through the heaviest R q-tiles, then through the next R, and so on; R is at most half
-      // the q-tiles of a head (a power of two up to 32), so that the last tiers are light ones and the compute units
-      // finish together.  Long sequences get R = 32: one head at a time.  The q-tiles of a head walk the same K/V
-      // tiles from tile 0 on at about the same pace, so one of them fetches a tile into the XCD's L2 and the others
-      // hit it there (a quarter of the L2 fills of the plain heaviest-first order, where an XCD works on all its heads
-      // at once), and neighbouring q-tiles read neighbouring rows of Q.
-      const int x = blockIdx.x & 7, l = blockIdx.x >> 3, hpx = U >> 3;   // XCD, index inside it, heads per XCD
+      // neighbouring q-tiles of FEW heads: the q-tiles of a head (by weight: rank 0 is the heaviest) are cut into ranges
+      // of R consecutive ranks, and the XCD goes through a range head by head, a head's R q-tiles in a row, before it
+      // moves on to the next range; 32 consecutive workgroups are therefore R q-tiles of each of 32 / R heads.  R is a
+      // power of two up to 32 and at most half of a head's q-tiles (long sequences: 32, one head at a time).  The q-tiles
+      // of a head walk the same K/V tiles from tile 0 on at about the same pace, so one of them fetches a tile into the
+      // XCD's L2 and the others hit it there (a quarter of the L2 fills of the plain heaviest-first order, where an XCD
+      // works on all its heads at once), and neighbouring q-tiles read neighbouring rows of Q.
+      const int x = blockIdx.x & 7, hpx = U >> 3;   // XCD, heads per XCD
+      int l = blockIdx.x >> 3;                      // index inside the XCD
       int R = 32;
       while (R > 1 && 2 * R > a.nqt) R >>= 1;
-      const int Hg = 32 / R;
-      const int nfull = a.nqt / R, lfull = nfull * R * hpx;
-      int t, Rt, lr;                                                      // range of ranks, its size, index inside it
-      if (l < lfull) { t = l / (R * hpx); Rt = R; lr = l % (R * hpx); }
-      else { t = nfull; Rt = a.nqt - nfull * R; lr = l - lfull; }
-      const int gidx = lr / (Rt * Hg), rem = lr % (Rt * Hg);              // head group, index inside it (head-major)
-      rank = t * R + rem % Rt;
-      s = x + 8 * (gidx * Hg + rem / Rt);
+      if constexpr (CAUSAL) {
+        // Causal q-tiles get lighter with their rank, and the ranges narrower: never more than half of the ranks that
+        // are left (64 q-tiles: 32, 16, 8, 4, 2, 1, 1), so that the workgroups an XCD runs last are all short ones
+        // (+2.5 % on 64 x 32 heads of 1024 rows, nothing on long sequences).
+        int r0 = 0;
+        for (;;) {
+          while (R > 1 && 2 * R > a.nqt - r0) R >>= 1;
+          if (l < R * hpx) break;
+          l -= R * hpx;
+          r0 += R;
+          if (r0 >= a.nqt) return;   // (a grid larger than the tile count: nothing to do)
+        }
+        rank = r0 + l % R;
+        s = x + 8 * (l / R);
+      } else {
+        // all q-tiles cost the same: ranges of R ranks and one last range with the remainder
+        const int nfull = a.nqt / R, lfull = nfull * R * hpx;
+        int t, Rt, lr;                              // range, its width, index inside it
+        if (l < lfull) { t = l / (R * hpx); Rt = R; lr = l % (R * hpx); }
+        else { t = nfull; Rt = a.nqt - nfull * R; lr = l - lfull; }
+        rank = t * R + lr % Rt;
+        s = x + 8 * (lr / Rt);
+      }
     } else
 #endif
     { rank = blockIdx.x / U; s = blockIdx.x % U; }
