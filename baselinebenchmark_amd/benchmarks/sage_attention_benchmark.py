@@ -52,6 +52,10 @@ def build_parser() -> argparse.ArgumentParser:
     p.add_argument("--pv", choices=("fp16", "fp8"), default="fp16", help="precision of the P.V product")
     p.add_argument("--blkq", type=int, choices=(16, 32, 64, 128), default=128)
     p.add_argument("--blkk", type=int, choices=(16, 32, 64, 128), default=64)
+    p.add_argument("--q-interleave", type=int, choices=(1, 8), default=1,
+                   help="8: eight interleaved scales per Q block (rows r, r+8, ... share one: upstream's per-thread Q granularity)")
+    p.add_argument("--k-interleave", type=int, choices=(1, 4), default=1,
+                   help="4: four interleaved scales per K block (keys n with equal (n %% 8) // 2 share one; K blocks of 32+ keys)")
     p.add_argument("--warmup", type=int, default=5)
     p.add_argument("--rep", type=int, default=20)
     g = p.add_mutually_exclusive_group()
@@ -84,6 +88,8 @@ def validate(args) -> None:
         raise ValueError("num-kv-heads must divide num-heads")
     if args.atol < 0 or args.rtol < 0:
         raise ValueError("atol and rtol must be non-negative")
+    if args.k_interleave == 4 and args.blkk == 16:
+        raise ValueError("four interleaved K scales need K blocks of 32, 64 or 128 keys")
 
 
 def effective_ops(batch, heads, seq, dim, causal) -> float:
@@ -110,7 +116,8 @@ def run_isolated(args) -> None:
         cmd = [sys.executable, "-m", "baselinebenchmark_amd.benchmarks.sage_attention_benchmark", "--custom-shapes",
                "--path", args.path, "--batch-size", str(b), "--num-heads", str(hq), "--num-kv-heads", str(hkv),
                "--head-dim", str(d), "--seq-lens", str(t), "--dtype", dt, "--pv", args.pv, "--blkq", str(args.blkq),
-               "--blkk", str(args.blkk), "--warmup", str(args.warmup), "--rep", str(args.rep), "--atol", str(args.atol),
+               "--blkk", str(args.blkk), "--q-interleave", str(args.q_interleave), "--k-interleave", str(args.k_interleave),
+               "--warmup", str(args.warmup), "--rep", str(args.rep), "--atol", str(args.atol),
                "--rtol", str(args.rtol), "--seed", str(args.seed), "--results-dir", args.results_dir,
                "--check-reference" if args.check_reference else "--no-check-reference"]
         if args.causal:
@@ -121,21 +128,30 @@ def run_isolated(args) -> None:
 # ------------------------------------------------------------------------------------------------
 # everything below touches torch / the GPU
 # ------------------------------------------------------------------------------------------------
-def _quantised_inputs(torch, b, hq, hkv, t, d, blkq, blkk, dev):
+def _quantised_inputs(torch, b, hq, hkv, t, d, blkq, blkk, dev, qg=1, kg=1):
     """Synthetic operands of the reference table: small INT8 values, random scales, N(0,1) V."""
     q = torch.randint(-16, 16, (b, hq, t, d), device=dev, dtype=torch.int8)
     k = torch.randint(-16, 16, (b, hkv, t, d), device=dev, dtype=torch.int8)
     v = torch.randn((b, hkv, t, d), device=dev, dtype=torch.float16)
-    qs = 0.005 + 0.015 * torch.rand((b, hq, -(-t // blkq)), device=dev, dtype=torch.float32)
-    ks = 0.005 + 0.015 * torch.rand((b, hkv, -(-t // blkk)), device=dev, dtype=torch.float32)
+    qs = 0.005 + 0.015 * torch.rand((b, hq, -(-t // blkq) * qg), device=dev, dtype=torch.float32)
+    ks = 0.005 + 0.015 * torch.rand((b, hkv, -(-t // blkk) * kg), device=dev, dtype=torch.float32)
     return q, k, v, qs, ks
 
 
-def _formula_on_cpu(torch, q, k, v, qs, ks, blkq, blkk, causal):
+def _expand(torch, scale, blk, groups, length):
+    """Per-row scales from per-block ones; with interleaved scales row n takes scale (n // blk) * groups + its group."""
+    if groups == 1:
+        return scale.cpu().repeat_interleave(blk, dim=-1)[..., :length, None]
+    n = torch.arange(length)
+    g = n % 8 if groups == 8 else (n % 8) // 2
+    return scale.cpu()[..., (n // blk) * groups + g, None]
+
+
+def _formula_on_cpu(torch, q, k, v, qs, ks, blkq, blkk, causal, qg=1, kg=1):
     """softmax(ln2 * (q*qs)(k*ks)^T) v in fp32 on the host: the gate's yardstick."""
     q, k, v = q.cpu().float(), k.cpu().float(), v.cpu().float()
-    q = q * qs.cpu().repeat_interleave(blkq, dim=-1)[..., : q.shape[-2], None]
-    k = k * ks.cpu().repeat_interleave(blkk, dim=-1)[..., : k.shape[-2], None]
+    q = q * _expand(torch, qs, blkq, qg, q.shape[-2])
+    k = k * _expand(torch, ks, blkk, kg, k.shape[-2])
     g = q.shape[1] // k.shape[1]
     k, v = k.repeat_interleave(g, dim=1), v.repeat_interleave(g, dim=1)
     logits = torch.matmul(q, k.transpose(-1, -2)) * math.log(2.0)
@@ -155,11 +171,12 @@ def reference_gate(torch, sa, hq, hkv, d, out_dtype, args):
     q = torch.randint(-8, 8, (1, ghq, GATE_Q_LEN, d), device=dev, dtype=torch.int8)
     k = torch.randint(-8, 8, (1, gkv, GATE_KV_LEN, d), device=dev, dtype=torch.int8)
     v = torch.randn((1, gkv, GATE_KV_LEN, d), device=dev, dtype=torch.float16)
-    qs = 0.005 + 0.015 * torch.rand((1, ghq, -(-GATE_Q_LEN // args.blkq)), device=dev, dtype=torch.float32)
-    ks = 0.005 + 0.015 * torch.rand((1, gkv, -(-GATE_KV_LEN // args.blkk)), device=dev, dtype=torch.float32)
+    qg, kg = args.q_interleave, args.k_interleave
+    qs = 0.005 + 0.015 * torch.rand((1, ghq, -(-GATE_Q_LEN // args.blkq) * qg), device=dev, dtype=torch.float32)
+    ks = 0.005 + 0.015 * torch.rand((1, gkv, -(-GATE_KV_LEN // args.blkk) * kg), device=dev, dtype=torch.float32)
     out, _ = sa.forward(q, k, v, qs, ks, output_dtype=out_dtype, BLKQ=args.blkq, BLKK=args.blkk, is_causal=args.causal,
-                        pv_mode=args.pv)
-    expected = _formula_on_cpu(torch, q, k, v, qs, ks, args.blkq, args.blkk, args.causal)
+                        pv_mode=args.pv, q_interleave=qg, k_interleave=kg)
+    expected = _formula_on_cpu(torch, q, k, v, qs, ks, args.blkq, args.blkk, args.causal, qg, kg)
     actual = out.cpu().float()
     max_abs = (actual - expected).abs().max().item()
     if args.pv == "fp8":
@@ -237,15 +254,17 @@ def benchmark(args) -> list:
                 print("\t".join(str(rows[-1][c]) for c in COLUMNS), flush=True)
                 continue
             if path == "core":
-                q, k, v, qs, ks = _quantised_inputs(torch, b, hq, hkv, t, d, args.blkq, args.blkk, "cuda")
+                q, k, v, qs, ks = _quantised_inputs(torch, b, hq, hkv, t, d, args.blkq, args.blkk, "cuda", args.q_interleave,
+                                                    args.k_interleave)
                 fn = lambda: sa.forward(q, k, v, qs, ks, output_dtype=dtype, BLKQ=args.blkq, BLKK=args.blkk,  # noqa: E731
-                                        is_causal=args.causal, pv_mode=args.pv)
+                                        is_causal=args.causal, pv_mode=args.pv, q_interleave=args.q_interleave,
+                                        k_interleave=args.k_interleave)
             else:
                 q = torch.randn((b, hq, t, d), device="cuda", dtype=dtype)
                 k = torch.randn((b, hkv, t, d), device="cuda", dtype=dtype)
                 v = torch.randn((b, hkv, t, d), device="cuda", dtype=dtype)
                 fn = lambda: sa.sageattn(q, k, v, is_causal=args.causal, pv_mode=args.pv, BLKQ=args.blkq,  # noqa: E731
-                                         BLKK=args.blkk)
+                                         BLKK=args.blkk, q_interleave=args.q_interleave, k_interleave=args.k_interleave)
             stats = _time(torch, fn, args.warmup, args.rep)
             tflops = effective_ops(b, hq, t, d, args.causal) / stats["mean_ms"] * 1e-9
             rows.append({**base, "latency_ms": f"{stats['mean_ms']:.4f}", "median_ms": f"{stats['median_ms']:.4f}",

@@ -37,6 +37,9 @@ def test_custom_shapes_and_validation():
         bench.validate(p.parse_args(["--atol", "-1"]))
     with pytest.raises(SystemExit):
         p.parse_args(["--head-dim", "96"])
+    with pytest.raises(ValueError):
+        bench.validate(p.parse_args(["--blkk", "16", "--k-interleave", "4"]))
+    bench.validate(p.parse_args(["--blkq", "32", "--q-interleave", "8", "--k-interleave", "4"]))
 
 
 def test_ops_formula_and_statistics():
@@ -64,6 +67,13 @@ def test_tiny_run_gates_then_times_and_writes_a_result_file(tmp_path):
     for key in ("backend", "device", "operator", "framework_version", "driver_version", "commit", "cases", "tolerance"):
         assert key in doc
     assert doc["cases"][0]["shape"] == [1, 4, 256, 64] and doc["cases"][0]["warmup"] == 1
+    # upstream's per-thread granularities through the same gate and both paths
+    args = bench.build_parser().parse_args(["--custom-shapes", "--path", "both", "--batch-size", "1", "--num-heads", "4",
+                                            "--num-kv-heads", "2", "--head-dim", "128", "--seq-lens", "300", "--warmup", "1",
+                                            "--rep", "2", "--blkq", "32", "--q-interleave", "8", "--k-interleave", "4", "--pv", "fp8",
+                                            "--causal", "--results-dir", ""])
+    rows = bench.benchmark(args)
+    assert [r["status"] for r in rows] == ["PASS", "PASS"]
 
 
 @pytest.mark.gpu
