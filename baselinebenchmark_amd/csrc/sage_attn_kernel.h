@@ -33,19 +33,11 @@
 #include "sage_launch.h"
 #include <atomic>
 #include <cstdlib>
+// Tuning constants of the matrix phase (measured: one more or one fewer fragment ahead is within +-1 %).
+#define SAGE_KPF 4   // K fragments read ahead of the Q.K^T MFMA that consumes them
+#define SAGE_VPF 3   // V fragment pairs read ahead of the P.V MFMA that consumes them
 // Bit of the wavefront index that picks the group: wavefronts w and w + 4 share a SIMD.
-#ifndef SAGE_KPF
-#define SAGE_KPF 4
-#endif
-#ifndef SAGE_VPF
-#define SAGE_VPF 3
-#endif
-#ifndef SAGE_REQ_GROUP
-#define SAGE_REQ_GROUP 0
-#endif
-#ifndef SAGE_GSH
 #define SAGE_GSH 2
-#endif
 
 namespace sage {
 
@@ -195,7 +187,6 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
   else {
     const int U = a.B * a.Hq;
     NG = a.B * a.Hkv;
-#ifndef SAGE_RANK_MAJOR
     // (Causal problems with fewer than 16 q-tiles per compute unit keep the plain heaviest-first order: with so few
     // rounds the balance of the last one matters more than locality -- 5 % on 4 x 32 heads of 4096 rows.)
     if ((U & 7) == 0 && (NG & 7) == 0 && (!CAUSAL || a.nqt * (U >> 3) >= 512)) {
@@ -234,9 +225,9 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
         rank = t * R + lr % Rt;
         s = x + 8 * (lr / Rt);
       }
-    } else
-#endif
-    { rank = blockIdx.x / U; s = blockIdx.x % U; }
+    } else {
+      rank = blockIdx.x / U; s = blockIdx.x % U;
+    }
   }
   int gi, g;
   if ((NG & 7) == 0) { int x = s & 7, y = s >> 3; gi = x + 8 * (y / G); g = y % G; }
@@ -829,20 +820,15 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
     auto issuer_in_flight = [&](int j) {
       return j == 0 ? first_in_flight : LEAD == 1 ? 0 : (j + 1 < ntiles ? NK : 0) + (j < ntiles ? NV : 0);
     };
-#ifdef SAGE_NO_ODD_BARRIER
-    auto odd_barrier = [&]() {};
-#else
     auto odd_barrier = [&]() { lds_barrier(); };
-#endif
     if constexpr (VECMAX) {
-      // FP8 P.V: the matrix phase is nothing but MFMAs and their LDS reads (P.V of the previous tile, Q.K^T of the
+      // FP8 P.V, and FP16 P.V of head_dim 128: the matrix phase is nothing but MFMAs and their LDS reads (P.V of the previous tile, Q.K^T of the
       // next); the row maximum and the probabilities belong to the vector phase, which is the longer one.  Group 0
       // issues the tile requests of the period, for both wavefronts of each SIMD pair, after its last Q.K^T MFMA: a
       // request holds up the wavefront that issues it for 40-50 ns (in-kernel timers; a burst, the same requests
       // spread over the phase, shared between the groups or staggered by SIMD all cost the same per request), and
       // the end of group 0's matrix phase is where a wavefront would otherwise wait at the barrier for group 1's
-      // softmax (SAGE_REQ_GROUP=1 puts them at the end of group 1's vector phase instead: 1-3 % slower).
-#if SAGE_REQ_GROUP == 0
+      // softmax (at the end of group 1's vector phase instead they measured 1-3 % slower).
       if (grp == 0) {
         for (int j = 0; j <= ntiles; j++) {
           SAGE_PH(3);
@@ -871,36 +857,8 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
           if (j < wnt) qk(j);
         }
       }
-#else
-      if (grp == 0) {
-        for (int j = 0; j <= ntiles; j++) {
-          SAGE_PH(3);
-          even_barrier(j, j == 0 ? first_in_flight : 0);
-          SAGE_PH(0);
-          if (j >= 1 && j - 1 < wnt) pv(j - 1);
-          if (j < wnt) qk(j);
-          SAGE_PH(1);
-          odd_barrier();
-          SAGE_PH(2);
-          if (j < wnt) { rowmax(j); softmax(j); }
-        }
-      } else {
-        for (int j = 0; j <= ntiles; j++) {
-          SAGE_PH(3);
-          even_barrier(j, issuer_in_flight(j));
-          SAGE_PH(0);
-          if (j >= 1 && j - 1 < wnt) { rowmax(j - 1); softmax(j - 1); }
-          request_tiles(j);
-          SAGE_PH(1);
-          odd_barrier();
-          SAGE_PH(2);
-          if (j >= 1 && j - 1 < wnt) pv(j - 1);
-          if (j < wnt) qk(j);
-        }
-      }
-#endif
     } else if (grp == 0) {
-      // FP16 P.V.  The even phase is as long as group 1's softmax, which must not start late: all tile loads of
+      // FP16 P.V of head_dim 64.  The even phase is as long as group 1's softmax, which must not start late: all tile loads of
       // the period are issued here, by the group whose matrix phase has slack, after its P.V.
       for (int j = 0; j <= ntiles; j++) {
         even_barrier(j, issuer_in_flight(j));
