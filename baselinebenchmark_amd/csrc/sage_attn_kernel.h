@@ -25,10 +25,12 @@
 //     requests two tile periods ahead for FP8 P.V, two slots and one period for FP16 P.V.  The raw q-tile of
 //     the variants that quantise their own Q and the V scales of the epilogue arrive the same way, and the
 //     output leaves through an LDS transposition as whole rows.
-//   * The wavefronts of a workgroup form two groups that run half a tile apart, two barriers per tile:
-//     while one group feeds the matrix pipe (P.V of its last tile, Q.K^T of its next) the other runs
-//     the softmax of the tile in between on the vector ALU.  Wavefronts w and w+4 share a SIMD and
-//     are in different groups, so each SIMD always has matrix work and vector work to overlap.
+//   * The wavefronts of a workgroup form two groups that run half a tile apart: while one group feeds the
+//     matrix pipe (P.V of its last tile, Q.K^T of its next) the other runs the softmax of the tile in
+//     between on the vector ALU.  Wavefronts w and w+4 share a SIMD and are in different groups, so each
+//     SIMD always has matrix work and vector work to overlap.  One barrier per tile period hands the tile
+//     slots over; the FP16 P.V kernels keep a second one in the middle of the period (their two slots are
+//     what it protects the pace of), the FP8 P.V kernels, with four slots, run their two halves unsynchronised.
 #pragma once
 #include "sage_launch.h"
 #include <atomic>
@@ -820,7 +822,11 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
     auto issuer_in_flight = [&](int j) {
       return j == 0 ? first_in_flight : LEAD == 1 ? 0 : (j + 1 < ntiles ? NK : 0) + (j < ntiles ? NV : 0);
     };
-    auto odd_barrier = [&]() { lds_barrier(); };
+    // The barrier in the middle of a period only keeps the two groups in step (no tile slot changes hands there: a
+    // period's requests go to slots whose last readers finished before the even barrier).  FP8 P.V kernels run without
+    // it: a group that finishes its half early starts the other half at once (+1.5 % at head_dim 128, +6 % at
+    // head_dim 64, where the vector half is much the longer one); FP16 P.V kernels measured equal or slower without.
+    auto odd_barrier = [&]() { if constexpr (PV == 0) lds_barrier(); };
     if constexpr (VECMAX) {
       // FP8 P.V, and FP16 P.V of head_dim 128: the matrix phase is nothing but MFMAs and their LDS reads (P.V of the previous tile, Q.K^T of the
       // next); the row maximum and the probabilities belong to the vector phase, which is the longer one.  Group 0
