@@ -804,6 +804,11 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
     // group 1's wavefronts to group 1, which requests them at the start of its matrix phase: both matrix phases then
     // carry part of the requests instead of one carrying all of them (+2 % from 4k to 16k keys).
     constexpr bool SPLIT_REQ = PV == 0 && VECMAX;
+    // FP8 kernels: group 0 requests the K tile of the period (after its matrix half), group 1 the V tile, as the first
+    // thing it does in the period: group 0's period (matrix half, requests, vector half) is the longer one, and V
+    // requests at any other place of group 1's period, or the K requests there, measured slower (+1.4 % for this one on
+    // config 2, +1.7 % on config 3, +3 % at head_dim 64).
+    constexpr bool V_BY_GROUP1 = PV == 1 && LEAD == 2;
     static_assert(!SPLIT_REQ || LEAD == 1, "group 1 requests V(j) in period j");
     auto first_value_tile = [&]() { load_v(0, 0); load_v(0, PARTNER); };
     auto request_tiles = [&](int j, bool with_first_value = true) {
@@ -813,14 +818,14 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
 #endif
       if (LEAD == 2 && j == 0 && with_first_value) first_value_tile();
       if (j + LEAD < ntiles) { load_k(j + LEAD, 0); load_k(j + LEAD, PARTNER); }
-      if (j + LEAD - 1 < ntiles) { load_v(j + LEAD - 1, 0); if (!SPLIT_REQ) load_v(j + LEAD - 1, PARTNER); }
+      if (!V_BY_GROUP1 && j + LEAD - 1 < ntiles) { load_v(j + LEAD - 1, 0); if (!SPLIT_REQ) load_v(j + LEAD - 1, PARTNER); }
 #ifdef SAGE_TIMING
       rq_sum += __builtin_amdgcn_s_memrealtime() - rq0;   // ticks this wavefront spent issuing the requests of a period
       rq_n++;
 #endif
     };
     auto issuer_in_flight = [&](int j) {
-      return j == 0 ? first_in_flight : LEAD == 1 ? 0 : (j + 1 < ntiles ? NK : 0) + (j < ntiles ? NV : 0);
+      return j == 0 ? first_in_flight : LEAD == 1 ? 0 : (j + 1 < ntiles ? NK : 0) + (!V_BY_GROUP1 && j < ntiles ? NV : 0);
     };
     // The barrier in the middle of a period only keeps the two groups in step (no tile slot changes hands there: a
     // period's requests go to slots whose last readers finished before the even barrier).  FP8 P.V kernels run without
@@ -828,13 +833,10 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
     // head_dim 64, where the vector half is much the longer one); FP16 P.V kernels measured equal or slower without.
     auto odd_barrier = [&]() { if constexpr (PV == 0) lds_barrier(); };
     if constexpr (VECMAX) {
-      // FP8 P.V, and FP16 P.V of head_dim 128: the matrix phase is nothing but MFMAs and their LDS reads (P.V of the previous tile, Q.K^T of the
-      // next); the row maximum and the probabilities belong to the vector phase, which is the longer one.  Group 0
-      // issues the tile requests of the period, for both wavefronts of each SIMD pair, after its last Q.K^T MFMA: a
-      // request holds up the wavefront that issues it for 40-50 ns (in-kernel timers; a burst, the same requests
-      // spread over the phase, shared between the groups or staggered by SIMD all cost the same per request), and
-      // the end of group 0's matrix phase is where a wavefront would otherwise wait at the barrier for group 1's
-      // softmax (at the end of group 1's vector phase instead they measured 1-3 % slower).
+      // FP8 P.V, and FP16 P.V of head_dim 128: the matrix half is nothing but MFMAs and their LDS reads (P.V of the
+      // previous tile, Q.K^T of the next); the row maximum and the probabilities belong to the vector half.  Group 0
+      // issues its tile requests, for both wavefronts of each SIMD pair, after its last Q.K^T MFMA (a request holds up
+      // the wavefront that issues it for 40-50 ns); group 1 issues its share as said above.
       if (grp == 0) {
         for (int j = 0; j <= ntiles; j++) {
           SAGE_PH(3);
@@ -852,8 +854,10 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
       } else {
         for (int j = 0; j <= ntiles; j++) {
           SAGE_PH(3);
-          even_barrier(j, j == 0 ? first_in_flight : 0);
+          // (the V tile requested a period ago, for the next period, may still be in flight)
+          even_barrier(j, j == 0 ? first_in_flight : (V_BY_GROUP1 && j < ntiles ? NV : 0));
           SAGE_PH(0);
+          if (V_BY_GROUP1 && j + 1 < ntiles) { load_v(j + 1, 0); load_v(j + 1, PARTNER); }
           if (j >= 1 && j - 1 < wnt) { rowmax(j - 1); softmax(j - 1); }
           SAGE_PH(1);
           odd_barrier();
