@@ -133,10 +133,12 @@ hipError_t launch_attn(const AttnArgs& a, int D, int pv, bool causal, int grid, 
   if (a.k_interleave) return launch_attn_kinterleaved(a, D, pv, causal, grid, st);
   if (a.blkk == 16) return launch_attn_k16(a, D, pv, causal, grid, st);
   if (a.q_raw) return launch_attn_qfused(a, D, pv, causal, grid, st);
-  const bool msum = pv && a.lse == nullptr;   // row sums on the matrix pipe unless LSE is wanted
+  // Row sums on the matrix pipe unless LSE is wanted (FP16 P.V: only head_dim 64 gains by it; head_dim 128 is
+  // bound by its matrix phases and keeps the sums on the vector ALU).
+  const bool msum = a.lse == nullptr;
 #define SAGE_ATTN(DD, PVV, BNN, MS) (causal ? launch_one<DD, 8, BNN, PVV, true, MS, 0>(a, grid, st) : launch_one<DD, 8, BNN, PVV, false, MS, 0>(a, grid, st))
   if (D == 128) return pv ? (msum ? SAGE_ATTN(128, 1, 128, true) : SAGE_ATTN(128, 1, 128, false)) : SAGE_ATTN(128, 0, 128, false);
-  return pv ? (msum ? SAGE_ATTN(64, 1, 128, true) : SAGE_ATTN(64, 1, 128, false)) : SAGE_ATTN(64, 0, 128, false);
+  return pv ? (msum ? SAGE_ATTN(64, 1, 128, true) : SAGE_ATTN(64, 1, 128, false)) : (msum ? SAGE_ATTN(64, 0, 128, true) : SAGE_ATTN(64, 0, 128, false));
 #undef SAGE_ATTN
 }
 

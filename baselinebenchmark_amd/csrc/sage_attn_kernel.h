@@ -161,8 +161,9 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
   constexpr int NSLOT = attn_tile_slots<PV, CAUSAL>(), LEAD = attn_tile_lead<PV, CAUSAL>();   // tiles are requested LEAD periods ahead
   // FP8 P.V: the softmax denominator of O always comes from the matrix pipe (the sum of the very fp8 values that
   // multiply V); MSUM additionally means that no fp32 sum is kept (no LSE wanted), and then the probabilities are
-  // coded without v_exp_f32 (FASTP, see softmax).
-  constexpr bool RSUM = PV == 1;
+  // coded without v_exp_f32 (FASTP, see softmax).  FP16 P.V kernels instantiated with MSUM (no LSE wanted) take the sum
+  // of the fp16-rounded probabilities from the matrix pipe as well; otherwise they sum in fp32 on the vector ALU.
+  constexpr bool RSUM = PV == 1 || MSUM;
   constexpr bool FASTP = PV == 1 && MSUM && MASK == 0;
   // FP8 kernels, and FP16 ones of head_dim 128, take the row maximum in the vector phase and issue the tile requests at
   // the end of group 0's matrix phase; FP16 kernels of head_dim 64 keep the row maximum in the matrix phase (their
@@ -458,17 +459,24 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
 #pragma unroll
     for (int i = 0; i < 16; i++) o[dt][i] = 0.f;
   float m_used = kMInit, lsum = 0.f;
-  // FP8 P.V: the row sums come out of the matrix pipe too.  A V^T operand of all ones (fp8 1.0 = 0x38)
-  // makes every row of one extra 32x32 output tile equal to sum_n P[n][m], i.e. the softmax
-  // denominator of query row m -- of the very fp8 values that multiply V.  The sum of rounded
+  // FP8 P.V: the row sums come out of the matrix pipe too, from one 16x16x128 MFMA (8 passes, half the time of
+  // a P.V one) per 64 keys.  Its B operand is the very register block that multiplies V: read by that
+  // instruction, lane l holds 32 codes of "column" l % 16 and k-chunk l / 16, where the 32x32x64 layout has
+  // query column l % 32 and key half l / 32 -- so chunks 0 and 2 are the two key halves of query columns 0-15 and
+  // chunks 1 and 3 those of columns 16-31.  The A operand selects them: row 0 is ones (fp8 1.0 = 0x38) over chunks
+  // 0 and 2, row 4 over chunks 1 and 3, every other row zero.  Output row 0 lands in register 0 of lanes 0-15
+  // and row 4 in register 0 of lanes 16-31: register 0 of lane l < 32 accumulates sum_n P[n][l], the softmax
+  // denominator of the lane's own query row -- of the very fp8 values that multiply V.  The sum of rounded
   // values is the right denominator for O but costs LSE accuracy on rows with few keys, so kernels
   // that return LSE (MSUM false) also keep the fp32 sum of the unrounded values on the vector ALU, for LSE alone.
-  v16f osum;
-#pragma unroll
-  for (int i = 0; i < 16; i++) osum[i] = 0.f;
+  v4f osum = {0.f, 0.f, 0.f, 0.f};
+  // (FP16 P.V kernels that return no LSE do the same with a 16x16x32 MFMA per 16 keys: 8 halves per lane and chunk.)
   v8i ones;
+  {
+    const bool sel = lane == 0 || lane == 32 || lane == 20 || lane == 52;
 #pragma unroll
-  for (int i = 0; i < 8; i++) ones[i] = 0x38383838;
+    for (int i = 0; i < 8; i++) ones[i] = !sel ? 0 : PV == 1 ? 0x38383838 : 0x3c003c00;
+  }
   asm volatile("" : "+v"(ones));
 
   // State that crosses phases: the raw scores of the tile in flight, its row maximum and scales, and
@@ -606,10 +614,7 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
       const float m_new = fmaxf(m_used, mall);
       const float alpha = __builtin_amdgcn_exp2f(m_used - m_new);
       lsum *= alpha;
-      if constexpr (RSUM) {
-#pragma unroll
-        for (int i = 0; i < 16; i++) osum[i] *= alpha;
-      }
+      if constexpr (RSUM) osum[0] *= alpha;
 #pragma unroll
       for (int dt = 0; dt < DTN; dt++)
 #pragma unroll
@@ -619,20 +624,25 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
     // P = exp2(S - m) * 2^PSHIFT, packed straight into the B operand of the second MFMA
     if constexpr (FASTP) {
       // The byte of an e4m3 number, read as an integer, is 8*(exponent + 7) + mantissa: piecewise linear in
-      // log2 of the value.  So u8(round(8*t + 56)) is the fp8 code of a number within a mantissa step of
-      // 2^t, with the mantissa interpolated linearly between powers of two instead of exponentially
-      // (kCodeBias centres the error of that, at most a third of a code step).  One v_fma_f32 and one
-      // v_cvt_pk_u8_f32 (round to nearest even, saturating at 0: masked scores are -inf and give +0) per
-      // score replace v_fma_f32 + v_exp_f32 + half a v_cvt_pk_fp8_f32: the vector ALU is the busier pipe.
+      // log2 of the value.  So y = 8*t + 56, rounded to an integer, is the fp8 code of a number within a mantissa
+      // step of 2^t, with the mantissa interpolated linearly between powers of two instead of exponentially
+      // (kCodeBias centres the error of that, at most a third of a code step).  Per score that is one v_fma_f32
+      // and three quarters of a conversion instead of v_fma_f32 + v_exp_f32 + half a v_cvt_pk_fp8_f32 (the
+      // vector ALU is the busier pipe): v_cvt_pknorm_u16_f32 turns two values x into round(65535 * x),
+      // saturating at 0 (masked scores are -inf and give code 0); with x = (256 * y + 127.5) / 65535, which the
+      // fma delivers directly, the high byte of each 16-bit result is y rounded to nearest, and one v_perm_b32
+      // gathers the high bytes of four results into a dword of the B operand.
       // t <= PSHIFT + TAU = 8, so the code stays <= 120 (= 256.0), below 0x7f.  The row sums of these very
       // codes come from the matrix pipe, so numerator and denominator of O see the same values.
-      const float k0 = 8.0f * (PSHIFT - m_used) + (56.0f + kCodeBias);
+      constexpr float kN = 256.0f / 65535.0f, kN8 = 8.0f * kN;
+      constexpr float kC = kN * (56.0f + kCodeBias) + 127.5f / 65535.0f;
+      const float k0 = __builtin_fmaf(kN8, PSHIFT - m_used, kC);
 #pragma unroll
       for (int nt = 0; nt < NT; nt++) {
         float c[SUBS], mul[SUBS];
 #pragma unroll
         for (int sub = 0; sub < SUBS; sub++) {
-          mul[sub] = 8.0f * sc[nt * SUBS + sub];
+          mul[sub] = kN8 * sc[nt * SUBS + sub];
           c[sub] = __builtin_fmaf(-kBiasF, mul[sub], k0);
         }
         float t8[16];
@@ -640,11 +650,9 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
         for (int r = 0; r < 16; r++) t8[r] = __builtin_fmaf(as_f(acc[nt][r]), mul[subof(r)], c[subof(r)]);
 #pragma unroll
         for (int q4 = 0; q4 < 4; q4++) {
-          // all four bytes get written, so the 'old' operand of the first insertion is a don't-care
-          unsigned d = (unsigned)acc[0][4 * nt + q4];
-#pragma unroll
-          for (int e = 0; e < 4; e++) d = __builtin_amdgcn_cvt_pk_u8_f32(t8[4 * q4 + e], e, d);
-          acc[0][4 * nt + q4] = (int)d;
+          const unsigned w01 = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_pknorm_u16(t8[4 * q4], t8[4 * q4 + 1]));
+          const unsigned w23 = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_pknorm_u16(t8[4 * q4 + 2], t8[4 * q4 + 3]));
+          acc[0][4 * nt + q4] = (int)__builtin_amdgcn_perm(w23, w01, 0x07050301u);
         }
       }
     } else if constexpr (PV == 1) {
@@ -687,8 +695,10 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
           v2f pp;
           pp[0] = __builtin_amdgcn_exp2f(__builtin_fmaf(as_f(acc[nt][r]), mul[subof(r)], c[subof(r)]));
           pp[1] = __builtin_amdgcn_exp2f(__builtin_fmaf(as_f(acc[nt][r + 1]), mul[subof(r)], c[subof(r)]));
-          lsum += pp[0];
-          lsum += pp[1];
+          if constexpr (!RSUM) {
+            lsum += pp[0];
+            lsum += pp[1];
+          }
           acc[nt][r >> 1] = __builtin_bit_cast(int, __builtin_convertvector(pp, v2h));
         }
       }
@@ -719,7 +729,7 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
 #pragma unroll
         for (int e = 0; e < 8; e++) pb[e] = acc[0][8 * kk + e];
         if constexpr (RSUM) {
-          if (dt == 0) osum = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ones, pb, osum, 0, 0, 0, 0, 0, 0);
+          if (dt == 0) osum = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ones, pb, osum, 0, 0, 0, 0, 0, 0);
         }
         o[dt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vf[i], pb, o[dt], 0, 0, 0, 0, 0, 0);
       }
@@ -742,11 +752,17 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
         if (i + VPF < NV) vf[i + VPF] = vfrag(i + VPF);
         const int nt = k16 >> 1, half = k16 & 1;
         const v4i pw = {acc[nt][4 * half], acc[nt][4 * half + 1], acc[nt][4 * half + 2], acc[nt][4 * half + 3]};
+        if constexpr (RSUM) {
+          const v4i oh = {ones[0], ones[1], ones[2], ones[3]};
+          if (dt == 0)
+            osum = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, oh), __builtin_bit_cast(v8h, pw), osum, 0, 0, 0);
+        }
         o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[i], __builtin_bit_cast(v8h, pw), o[dt], 0, 0, 0);
       }
       __builtin_amdgcn_sched_group_barrier(0x100, VPF, 0);
 #pragma unroll
       for (int i = 0; i < NV; i++) {
+        if (RSUM && i % DTN == 0) __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
         if (i + VPF < NV) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
       }
@@ -891,10 +907,13 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
   SAGE_T(5, lsum);   // main loop done
   // ---- epilogue: O = O^T / l (* v_scale), LSE2 = m + log2(l) ----
   // The denominator of O: FP8 kernels take the matrix pipe's sum of the rounded probabilities (already the full row
-  // sum: the MFMA contracts over both lane halves); the fp32 sum of the unrounded ones serves LSE only.
-  if constexpr (MSUM) lsum = osum[0];
+  // sum: the MFMA contracts over both key halves; it sits in lanes 0-31, lanes 32-63 hold zero and get it from
+  // their partner); the fp32 sum of the unrounded ones serves LSE only.
+  float msum = 0.f;
+  if constexpr (RSUM) msum = xchg32_sum(osum[0]);
+  if constexpr (MSUM) lsum = msum;
   else lsum = xchg32_sum(lsum);
-  const float den = RSUM ? osum[0] : lsum;
+  const float den = RSUM ? msum : lsum;
   const float inv = den > 0.f ? 1.0f / den : 0.f;   // a row with no visible key yields zeros
   if (my_row < Lq) {
     if (a.lse && h == 0) {

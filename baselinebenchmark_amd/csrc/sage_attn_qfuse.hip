@@ -7,10 +7,10 @@
 namespace sage {
 
 hipError_t launch_attn_qfused(const AttnArgs& a, int D, int pv, bool causal, int grid, hipStream_t st) {
-  const bool msum = pv && a.lse == nullptr;
+  const bool msum = a.lse == nullptr;
 #define SAGE_ATTN_Q(DD, PVV, BNN, MS) (causal ? launch_one<DD, 8, BNN, PVV, true, MS, 0, 1, true>(a, grid, st) : launch_one<DD, 8, BNN, PVV, false, MS, 0, 1, true>(a, grid, st))
   if (D == 128) return pv ? (msum ? SAGE_ATTN_Q(128, 1, 128, true) : SAGE_ATTN_Q(128, 1, 128, false)) : SAGE_ATTN_Q(128, 0, 128, false);
-  return pv ? (msum ? SAGE_ATTN_Q(64, 1, 128, true) : SAGE_ATTN_Q(64, 1, 128, false)) : SAGE_ATTN_Q(64, 0, 128, false);
+  return pv ? (msum ? SAGE_ATTN_Q(64, 1, 128, true) : SAGE_ATTN_Q(64, 1, 128, false)) : (msum ? SAGE_ATTN_Q(64, 0, 128, true) : SAGE_ATTN_Q(64, 0, 128, false));
 #undef SAGE_ATTN_Q
 }
 

@@ -12,7 +12,8 @@ output type instead:
     some row of its group grew by more than tau = 3 over it (lazy rescale), then o and the row sum are scaled by
     exp2(old - new);
   * P = 2^5 * exp2(s - m) rounded to e4m3 (round to nearest even) -- or, for the kernels that need no LSE and no
-    explicit mask, the "linear-mantissa" code u8(rne(8 * t + 56 - 0.3)), t = s - m + 5, read as an e4m3 byte;
+    explicit mask, the "linear-mantissa" code: 8 * t + 56 - 0.3, t = s - m + 5, rounded to nearest (as the high byte of a
+    16-bit conversion of (256 * code + 127.5) / 65535) and read as an e4m3 byte;
   * O = sum P8 * V8 and the denominator sum P8 (of the very same rounded values), fp32 accumulation on the GPU,
     float64 here; out = O / den * v_scale;  LSE2 = m + log2(sum of the unrounded p) - 5.
 
@@ -31,6 +32,9 @@ PSHIFT = np.float32(5.0)
 TAU = np.float32(3.0)
 CODE_BIAS = np.float32(-0.3)
 M_INIT = np.float32(-1.0e30)
+KN = np.float32(256.0) / np.float32(65535.0)                      # code units -> units of the 16-bit conversion
+KN8 = np.float32(8.0) * KN
+KC = np.float32(np.float32(KN * np.float32(np.float32(56.0) + CODE_BIAS)) + np.float32(127.5) / np.float32(65535.0))
 TILE = 128                         # keys per tile
 GROUP = 32                         # query rows per wavefront
 
@@ -45,6 +49,20 @@ def decode_e4m3(code: np.ndarray) -> np.ndarray:
     code = code.astype(np.int64)
     e, m = code >> 3, code & 7
     return np.where(e == 0, m * 2.0 ** -9, np.exp2((e - 7).astype(np.float64)) * (1.0 + m / 8.0))
+
+
+def linear_code_of(acc: np.ndarray, sc: np.ndarray, base: np.ndarray) -> np.ndarray:
+    """The kernel's linear-mantissa code of 2^t, t = (acc - BIAS) * sc + base: y = 8 * t + 56 + CODE_BIAS rounded to
+    nearest, computed the kernel's way (baselinebenchmark_amd/csrc/sage_attn_kernel.h, softmax): fp32 FMAs deliver
+    x = (256 * y + 127.5) / 65535, the 16-bit conversion gives rne(65535 * x) saturated to [0, 65535], and the code is
+    its high byte.  acc [R, N] biased fp32 accumulators, sc [R, N] fp32 scale products, base [R] fp32."""
+    k0 = _fma32(KN8, base, KC)
+    mul = (KN8 * sc).astype(np.float32)
+    c = _fma32(-BIAS, mul, k0[:, None])
+    x = _fma32(acc, mul, c)
+    with np.errstate(invalid="ignore"):
+        u16 = np.rint(np.clip(x.astype(np.float64), 0.0, 1.0) * 65535.0)
+    return np.floor(u16 / 256.0)
 
 
 def _rne_e4m3(p32: np.ndarray) -> np.ndarray:
@@ -125,11 +143,7 @@ def fp8_attention_model(q_int8, k_int8, v, q_scale, k_scale, tensor_layout="HND"
                 m_used = m_new
                 base = (PSHIFT - m_used).astype(np.float32)                       # [Sq]
                 if linear_code:
-                    k0 = (np.float32(8.0) * base + (np.float32(56.0) + CODE_BIAS)).astype(np.float32)
-                    mul = (np.float32(8.0) * sc).astype(np.float32)
-                    c = _fma32(-BIAS, mul, k0[:, None])
-                    t8 = _fma32(acc, mul, c)
-                    code = np.clip(np.rint(t8.astype(np.float64)), 0, 255)
+                    code = linear_code_of(acc, sc, base)
                     code = np.where(dead, 0, code)
                     p8 = decode_e4m3(code)
                 else:

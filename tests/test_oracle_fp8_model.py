@@ -45,6 +45,24 @@ def test_linear_code_is_within_a_mantissa_step_of_the_exponential():
     assert (np.diff(val) >= 0).all()                                                       # monotone
 
 
+def test_linear_code_by_way_of_the_16_bit_conversion_is_the_code_value_rounded_to_nearest():
+    """The kernel reaches the code through a 16-bit conversion and its high byte; away from ties that must be
+    rint(8 * t + 56 - 0.3) computed in float64 from the same operands, and next to ties one of the two neighbours."""
+    rng = np.random.default_rng(5)
+    R, N = 64, 128
+    dots = rng.integers(-40000, 40000, size=(R, N))
+    acc = (12582912.0 + dots).astype(np.float32)
+    sc = np.broadcast_to(rng.uniform(1e-4, 3e-4, size=(R, 1)).astype(np.float32), (R, N))
+    base = (5.0 - (dots.max(axis=1) * sc[:, 0].astype(np.float64))).astype(np.float32) + rng.uniform(0, 3, R).astype(np.float32)
+    code = fm.linear_code_of(acc, sc, base)
+    y = 8.0 * (dots * sc.astype(np.float64) + base[:, None].astype(np.float64)) + 56.0 - 0.3
+    want = np.clip(np.rint(y), 0, 255)
+    near_tie = np.abs(y - np.floor(y) - 0.5) < 0.02
+    assert (~near_tie).mean() > 0.9 and want.max() >= 100 and (want == 0).any()
+    assert (code[~near_tie] == want[~near_tie]).all()
+    assert (np.abs(code - want) <= 1).all()
+
+
 @pytest.mark.parametrize("linear", [False, True])
 def test_one_tile_closed_form_with_scalar_loops(linear):
     """Skv <= 128: one tile, the reference maximum is the row's own maximum, so the model must equal
