@@ -565,17 +565,30 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
     // ---- masking: only tiles that cross the diagonal or the end of the sequence ----
     const bool need_mask = (CAUSAL && (n0 + BN - 1 > row0)) || (n0 + BN > Lk);
     if (need_mask) {
+      // Register r of 32-key group nt holds key n0 + 32*nt + 8*(r/4) + r%4 + 4*h: it is masked when that index
+      // exceeds lim.  In causal kernels (two diagonal tiles per q-tile) the bounds of lim over the wavefront (its 32
+      // rows, both lane halves) sort the groups first: most are visible or masked as a whole, and only the one the
+      // diagonal runs through is selected element by element.
       const int lim = (CAUSAL ? min(my_row, Lk - 1) : Lk - 1) - n0 - 4 * h;
+      const int lim_hi = min(row0 + 31, Lk - 1) - n0, lim_lo = min(row0, Lk - 1) - n0 - 4;
 #pragma unroll
-      for (int nt = 0; nt < NT; nt++)
+      for (int nt = 0; nt < NT; nt++) {
+        if constexpr (CAUSAL) {
+          if (32 * nt + 27 <= lim_lo) continue;
+          if (32 * nt > lim_hi) {
 #pragma unroll
-        for (int r = 0; r < 16; r++)
-        {
-          // branch-free select on the sign of (lim - index): compare-and-select would hold 64 lane masks
+            for (int r = 0; r < 16; r++) acc[nt][r] = as_i(kNegInf);
+            continue;
+          }
+        }
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          // branch-free select on the sign of (lim - index): compare-and-select would hold the lane masks
           // in scalar registers at once
           const int gone = (lim - (32 * nt + 8 * (r / 4) + (r % 4))) >> 31;
           acc[nt][r] = (acc[nt][r] & ~gone) | (as_i(kNegInf) & gone);
         }
+      }
     }
     // ---- row maximum of this tile, in score units ----
     // The biased scores are positive floats (or -inf where masked), so their bit patterns order like
