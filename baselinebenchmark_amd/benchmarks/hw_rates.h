@@ -13,8 +13,9 @@
  *
  * sage_coexec: how much the matrix pipe and the vector ALU of a SIMD slow each other down.  Workgroups of eight
  * wavefronts (two per SIMD): wavefronts 0-3 issue MFMAs (mfma_kind 0 INT8 32x32x32, 1 FP8 32x32x64; 16 per iteration),
- * wavefronts 4-7 vector instructions (valu_kind 0 v_fma_f32, 1 v_cvt_pk_u8_f32, 2 v_max3_i32, 3 the mix of the FP8
- * softmax: 64 + 64 + 32 per iteration).  mode 1 runs the MFMA half alone, 2 the vector half alone, 3 both.
+ * wavefronts 4-7 vector instructions (valu_kind 0 v_fma_f32, 1 v_cvt_pk_u8_f32, 2 v_max3_i32, 3 a mix of the FP8
+ * softmax with one conversion per code: 64 + 64 + 32 per iteration, 4 the mix the kernels run: 64 v_fma_f32 +
+ * 32 v_cvt_pknorm_u16_f32 + 16 v_perm_b32 + 32 v_max3_i32).  mode 1 runs the MFMA half alone, 2 the vector half alone, 3 both.
  */
 #ifndef SAGE_HW_RATES_H
 #define SAGE_HW_RATES_H

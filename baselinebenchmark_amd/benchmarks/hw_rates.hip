@@ -116,7 +116,7 @@ __global__ void __launch_bounds__(1024) microbench_kernel(int* sink, int iters, 
 // Co-execution of the two pipes of a SIMD: a workgroup of eight wavefronts, two per SIMD; wavefronts 0-3 issue MFMAs
 // (MK 0: v_mfma_i32_32x32x32_i8, 1: v_mfma_f32_32x32x64_f8f6f4, four accumulators in turn), wavefronts 4-7 vector
 // instructions (VK 0: v_fma_f32, 1: v_cvt_pk_u8_f32, 2: v_max3_i32, 3: the mix of the FP8 softmax without v_exp_f32: per
-// 64 scores 64 fma + 64 cvt_pk_u8 + 32 max3).  mode bit 0 / 1 switches each half on: timing a half alone and both together
+// 64 scores 64 fma + 64 cvt_pk_u8 + 32 max3; 4: the mix the kernels run now, 64 fma + 32 cvt_pknorm_u16 + 16 perm + 32 max3).  mode bit 0 / 1 switches each half on: timing a half alone and both together
 // says how much the pipes slow each other down.  Per iteration: 16 MFMAs, or 64 / 64 / 32 / 160 vector instructions.
 template <int MK, int VK>
 __global__ void __launch_bounds__(512) coexec_kernel(int* sink, int iters, int mode, float s, float c) {
@@ -145,15 +145,23 @@ __global__ void __launch_bounds__(512) coexec_kernel(int* sink, int iters, int m
     for (int it = 0; it < iters; it++) {
 #pragma unroll
       for (int u = 0; u < 4; u++) {
-        if constexpr (VK == 0 || VK == 3) {
+        if constexpr (VK == 0 || VK == 3 || VK == 4) {
 #pragma unroll
           for (int i = 0; i < 16; i++) x[i] = __builtin_fmaf(x[i], s, c);
+        }
+        if constexpr (VK == 4) {   // two codes per conversion, one v_perm_b32 per four
+#pragma unroll
+          for (int i = 0; i < 16; i += 4) {
+            const unsigned w01 = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_pknorm_u16(x[i], x[i + 1]));
+            const unsigned w23 = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_pknorm_u16(x[i + 2], x[i + 3]));
+            pk[i >> 2] ^= __builtin_amdgcn_perm(w23, w01, 0x07050301u);
+          }
         }
         if constexpr (VK == 1 || VK == 3) {
 #pragma unroll
           for (int i = 0; i < 16; i++) pk[i >> 2] = __builtin_amdgcn_cvt_pk_u8_f32(x[i], i & 3, pk[i >> 2]);
         }
-        if constexpr (VK == 2 || VK == 3) {
+        if constexpr (VK == 2 || VK == 3 || VK == 4) {
 #pragma unroll
           for (int i = 0; i < 16; i += 2)
             mx[(i >> 1) & 3] = max(max(mx[(i >> 1) & 3], __builtin_bit_cast(int, x[i])), __builtin_bit_cast(int, x[i + 1]));
@@ -231,19 +239,19 @@ int sage_microbench(int kind, int grid, int waves_per_simd, int iters, void* sin
 }
 
 // Co-execution benchmark: `grid` workgroups of eight wavefronts, `iters` iterations; mfma_kind 0 (INT8) or 1 (FP8),
-// valu_kind 0 fma, 1 cvt_pk_u8, 2 max3, 3 the mix; mode 1 = the MFMA wavefronts only, 2 = the vector wavefronts only,
-// 3 = both.  Per iteration a wavefront issues 16 MFMAs, or 64 / 64 / 32 / 160 vector instructions.
+// valu_kind 0 fma, 1 cvt_pk_u8, 2 max3, 3 the mix with one conversion per code, 4 the mix with two per conversion; mode 1 = the MFMA wavefronts only, 2 = the vector wavefronts only,
+// 3 = both.  Per iteration a wavefront issues 16 MFMAs, or 64 / 64 / 32 / 160 / 144 vector instructions.
 int sage_coexec(int mfma_kind, int valu_kind, int mode, int grid, int iters, void* sink, size_t sink_bytes, void* stream) {
   using namespace sage;
-  if (mfma_kind < 0 || mfma_kind > 1 || valu_kind < 0 || valu_kind > 3 || mode < 1 || mode > 3) return HWR_EINVAL;
+  if (mfma_kind < 0 || mfma_kind > 1 || valu_kind < 0 || valu_kind > 4 || mode < 1 || mode > 3) return HWR_EINVAL;
   if (grid <= 0 || grid > 65535 || iters <= 0 || !sink) return HWR_EINVAL;
   if (sink_bytes < (size_t)grid * 1024 * sizeof(int)) return HWR_ESIZE;
   int* out = (int*)sink;
   hipStream_t st = (hipStream_t)stream;
   hipError_t e;
 #define SAGE_CX(M, V) launch_coexec<M, V>(out, grid, iters, mode, st)
-  if (mfma_kind == 0) e = valu_kind == 0 ? SAGE_CX(0, 0) : valu_kind == 1 ? SAGE_CX(0, 1) : valu_kind == 2 ? SAGE_CX(0, 2) : SAGE_CX(0, 3);
-  else e = valu_kind == 0 ? SAGE_CX(1, 0) : valu_kind == 1 ? SAGE_CX(1, 1) : valu_kind == 2 ? SAGE_CX(1, 2) : SAGE_CX(1, 3);
+  if (mfma_kind == 0) e = valu_kind == 0 ? SAGE_CX(0, 0) : valu_kind == 1 ? SAGE_CX(0, 1) : valu_kind == 2 ? SAGE_CX(0, 2) : valu_kind == 3 ? SAGE_CX(0, 3) : SAGE_CX(0, 4);
+  else e = valu_kind == 0 ? SAGE_CX(1, 0) : valu_kind == 1 ? SAGE_CX(1, 1) : valu_kind == 2 ? SAGE_CX(1, 2) : valu_kind == 3 ? SAGE_CX(1, 3) : SAGE_CX(1, 4);
 #undef SAGE_CX
   return e == hipSuccess ? HWR_OK : HWR_ELAUNCH;
 }

@@ -95,7 +95,8 @@ def run(iters_mfma: int = 4000, iters_valu: int = 20000) -> list[dict]:
 
 
 COEXEC_MFMA = ["v_mfma_i32_32x32x32_i8", "v_mfma_f32_32x32x64_f8f6f4 (fp8)"]
-COEXEC_VALU = [("v_fma_f32", 64), ("v_cvt_pk_u8_f32", 64), ("v_max3_i32", 32), ("softmax mix: 64 fma + 64 cvt_pk_u8 + 32 max3", 160)]
+COEXEC_VALU = [("v_fma_f32", 64), ("v_cvt_pk_u8_f32", 64), ("v_max3_i32", 32), ("softmax mix: 64 fma + 64 cvt_pk_u8 + 32 max3", 160),
+               ("softmax mix: 64 fma + 32 cvt_pknorm_u16 + 16 perm + 32 max3", 144)]
 
 
 def run_coexec(iters: int = 20000) -> list[dict]:
