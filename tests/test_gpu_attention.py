@@ -219,6 +219,34 @@ def test_lse_is_empty_unless_requested():
 
 
 @pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("shape", [(1, 2, 1, 129, 70), (2, 4, 2, 300, 1000), (1, 3, 3, 513, 513)])
+@pytest.mark.parametrize("D", [64, 128])
+def test_fp16_pv_without_lse_matches_the_reference_formula_and_the_lse_variant(D, shape, causal):
+    """Without LSE the FP16 P.V kernels of head_dim 64 take their row sums from the matrix pipe (the sum of the
+    fp16-rounded probabilities), with LSE from the vector ALU (the unrounded ones): two kernels, one formula.  Both must
+    meet the bound of the reference formula, and agree with each other to fp16 rounding of the output."""
+    B, Hq, Hkv, Sq, Skv = shape
+    if causal and Sq > Skv:
+        Sq = Skv
+    g = torch.Generator().manual_seed(77 + D + Sq)
+    q = randn("HND", B, Hq, Sq, D, torch.float16, g)
+    k = randn("HND", B, Hkv, Skv, D, torch.float16, g)
+    v = randn("HND", B, Hkv, Skv, D, torch.float16, g)
+    qi, qs, ki, ks = sa.per_block_int8(q.to(DEV), k.to(DEV), BLKQ=64, BLKK=64)
+    kw = dict(output_dtype=torch.float16, BLKQ=64, BLKK=64, is_causal=causal, pv_mode="fp16")
+    plain, none = sa.forward(qi, ki, v.to(DEV), qs, ks, **kw)
+    with_lse, lse = sa.forward(qi, ki, v.to(DEV), qs, ks, return_lse=True, **kw)
+    fused, _ = sa.forward_fused_q(q.to(DEV), ki, v.to(DEV), ks, **kw)
+    ref, _ = oa.sage_reference(qi.cpu(), ki.cpu(), v, qs.cpu(), ks.cpu(), "HND", 64, 64, is_causal=causal)
+    assert none.numel() == 0 and lse.numel() == B * Hq * Sq
+    for out in (plain, with_lse):
+        m = oa.metrics(out.cpu().float(), ref)
+        assert m["finite"] and m["rel_rmse"] < 2e-3, m
+    assert oa.metrics(plain.cpu().float(), with_lse.cpu().double())["rel_rmse"] < 6e-4
+    assert torch.equal(fused, plain)
+
+
+@pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("pv", ["fp16", "fp8"])
 @pytest.mark.parametrize("D", [64, 128])
 def test_k_scale_blocks_of_16_keys(causal, pv, D):
