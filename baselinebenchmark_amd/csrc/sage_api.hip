@@ -332,6 +332,10 @@ int sage_attn_fwd_masked(const int8_t* q, const int8_t* k, const void* v_panels,
 
 // ---- one-call pipeline --------------------------------------------------------------------
 namespace {
+// Up to this many keys per sequence and elements of K per call the pre-passes run as one launch whose workgroups read
+// their sequence's statistics themselves (sage_quant.hip: prepass_small_kernel).
+constexpr int kSmallPrepassRows = 1024;
+constexpr int64_t kSmallPrepassElements = (int64_t)4 << 20;
 struct E2EWorkspace {
   size_t q_i8, k_i8, q_scale, k_scale, km, v_scale, panels, stat, plan, lse_off, total;
   int64_t qs_sh, ks_sh, panel_sh;
@@ -436,13 +440,37 @@ int sage_sageattn_masked(const void* q, const void* k, const void* v, void* out,
   // and LSE = -inf without reading K, V or their scales.
   const bool no_keys = !varlen && Skv == 0;
   if (no_keys) smooth_k = 0;
-  if (smooth_k) {
-    rc = sage_k_mean(k, km, stat, stat_bytes, B, Hkv, Skv, D, k_sb, k_sh, k_sn, dtype, cu_seqlens_k, stream);
+  // Short sequences: all K and V pre-passes in one launch (every workgroup computes the statistic its tile needs over
+  // the whole sequence itself); otherwise six launches, the statistics in two stages.
+  const bool small_prepass = !varlen && !no_keys && Skv <= kSmallPrepassRows &&
+                             (int64_t)B * Hkv * Skv * D <= kSmallPrepassElements;
+  if (small_prepass) {
+    if (int rc2 = check_stride16("k", k_sb, k_sh, k_sn, 2, k)) return rc2;
+    if (int rc2 = check_stride16("v", v_sb, v_sh, v_sn, 2, v)) return rc2;
+    const int kb = blk_rows(blkk);
+    QuantArgs qa;
+    memset(&qa, 0, sizeof(qa));
+    qa.x = (const u16*)k; qa.out = k_i8; qa.scale = k_scale; qa.km = nullptr;
+    qa.B = B; qa.H = Hkv; qa.L = Skv; qa.D = D;
+    qa.x_sb = k_sb; qa.x_sh = k_sh; qa.x_sn = k_sn; qa.o_sb = ki_sb; qa.o_sh = ki_sh; qa.o_sn = ki_sn;
+    qa.blk = kb; qa.groups = blk_groups(blkk); qa.mult = 1.0f; qa.dv_group = 1;
+    PrepVArgs va;
+    memset(&va, 0, sizeof(va));
+    va.v = (const u16*)v; va.panels = (uint8_t*)panels; va.vscale = v_scale; va.B = B; va.H = Hkv; va.L = Skv; va.D = D;
+    va.v_sb = v_sb; va.v_sh = v_sh; va.v_sn = v_sn;
+    hipError_t e = launch_prepass_small(qa, va, dtype, pv_mode == SAGE_PV_FP8, (Skv + kb - 1) / kb,
+                                        (Skv + SAGE_PANEL_ROWS - 1) / SAGE_PANEL_ROWS, smooth_k != 0, km, v_scale,
+                                        (hipStream_t)stream);
+    if (e != hipSuccess) return hip_fail(e, "sage_sageattn(pre-pass)");
+  } else {
+    if (smooth_k) {
+      rc = sage_k_mean(k, km, stat, stat_bytes, B, Hkv, Skv, D, k_sb, k_sh, k_sn, dtype, cu_seqlens_k, stream);
+      if (rc) return rc;
+    }
+    if (!no_keys) rc = sage_quant_int8(k, k_i8, k_scale, smooth_k ? km : nullptr, B, Hkv, Skv, D, k_sb, k_sh, k_sn, ki_sb, ki_sh, ki_sn,
+                         (int64_t)Hkv * D, D, blkk, 1.0f, dtype, cu_seqlens_k, cu_kblk, w.ks_sh, stream);
     if (rc) return rc;
   }
-  if (!no_keys) rc = sage_quant_int8(k, k_i8, k_scale, smooth_k ? km : nullptr, B, Hkv, Skv, D, k_sb, k_sh, k_sn, ki_sb, ki_sh, ki_sn,
-                       (int64_t)Hkv * D, D, blkk, 1.0f, dtype, cu_seqlens_k, cu_kblk, w.ks_sh, stream);
-  if (rc) return rc;
   // With K smoothing every logit of a query row loses q . k_mean; the softmax does not notice but the
   // log-sum-exp does, so when LSE is requested the Q quantiser also emits that dot product (in the
   // base-2 units of the scaled Q) and the attention kernel adds it back.
@@ -461,7 +489,7 @@ int sage_sageattn_masked(const void* q, const void* k, const void* v, void* out,
                     cu_seqlens_q, cu_qblk, w.qs_sh, dot, stream);
     if (rc) return rc;
   }
-  if (!no_keys) {
+  if (!no_keys && !small_prepass) {
     rc = sage_prep_v(v, panels, v_scale, stat, stat_bytes, B, Hkv, Skv, D, v_sb, v_sh, v_sn, dtype, pv_mode, cu_seqlens_k,
                      cu_panel, w.panel_sh, stream);
     if (rc) return rc;

@@ -93,6 +93,10 @@ int colstat_chunks(int L);
 hipError_t launch_k_mean(const ColStatArgs& a, int dtype, void* km, hipStream_t st);
 hipError_t launch_v_scale(const ColStatArgs& a, int dtype, float* vscale, hipStream_t st);
 hipError_t launch_prep_v(const PrepVArgs& a, int dtype, int pv, int max_panels, hipStream_t st);
+// Short fixed-length sequences: K mean + K quantiser + V scale + V panels in one launch (nk K tiles and nv V panels per
+// (batch, kv-head); km_out / vscale_out take the statistics; qa.km is ignored and must be null).
+hipError_t launch_prepass_small(const QuantArgs& qa, const PrepVArgs& va, int dtype, int pv, int nk, int nv, int smooth,
+                                void* km_out, float* vscale_out, hipStream_t st);
 
 AttnConfig attn_config(int D, int pv, bool packed);
 hipError_t launch_attn(const AttnArgs& a, int D, int pv, bool causal, int grid, hipStream_t st);

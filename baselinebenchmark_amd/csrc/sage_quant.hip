@@ -17,12 +17,13 @@ namespace sage {
 // One workgroup (256 lanes) quantises one [blk, D] tile held entirely in registers:
 // pass 1 converts and reduces |x| to the tile maximum, pass 2 divides and rounds.
 // A lane owns 16 consecutive channels of a row (two 128-bit loads, one 128-bit store).
+// (km_lds: the K mean of this (batch, head) in LDS, D values in the input dtype, instead of a.km in global memory:
+// the fused pre-pass of short sequences computes it in the same workgroup.)
 template <int DT, int D>
-__global__ void __launch_bounds__(256) quant_int8_kernel(QuantArgs a) {
+__device__ __forceinline__ void quant_int8_tile(const QuantArgs& a, const int blkid, const int h, const int b, const u16* km_lds) {
   constexpr int TPR = D / 16;       // lanes per row
   constexpr int RPP = 256 / TPR;    // rows per pass
   constexpr int MAXP = 128 / RPP;   // passes for the largest tile (128 rows)
-  const int blkid = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
   const int tid = threadIdx.x;
   const int tr = tid / TPR, tc = tid % TPR;
 
@@ -46,8 +47,11 @@ __global__ void __launch_bounds__(256) quant_int8_kernel(QuantArgs a) {
   const int rows = min(a.blk, L - n0);
 
   float kmv[16];
-  const bool has_km = a.km != nullptr;
-  if (has_km) {
+  const bool has_km = a.km != nullptr || km_lds != nullptr;
+  if (km_lds) {
+#pragma unroll
+    for (int i = 0; i < 16; i++) kmv[i] = to_f32<DT>(km_lds[tc * 16 + i]);
+  } else if (has_km) {
     const uint4* kp = reinterpret_cast<const uint4*>(a.km + (int64_t)b * a.km_sb + (int64_t)h * a.km_sh + tc * 16);
     uint4 raw2[2] = {kp[0], kp[1]};
     const u16* p = reinterpret_cast<const u16*>(raw2);
@@ -162,6 +166,11 @@ __global__ void __launch_bounds__(256) quant_int8_kernel(QuantArgs a) {
   }
 }
 
+template <int DT, int D>
+__global__ void __launch_bounds__(256) quant_int8_kernel(QuantArgs a) {
+  quant_int8_tile<DT, D>(a, blockIdx.x, blockIdx.y, blockIdx.z, nullptr);
+}
+
 // ---------------------------------------------------------------------------------------------
 // Column statistics over the sequence: MODE 0 = float64 sum (K mean), MODE 1 = fp32 abs-max (V).
 // Stage 1: one workgroup per (chunk of kChunkRows rows, head, batch) writes D partials.
@@ -265,8 +274,9 @@ __global__ void vscale_finalize_kernel(const float* partial, float* vscale, int 
 // Elements are converted, scattered into LDS in panel byte order and streamed out linearly.
 // ---------------------------------------------------------------------------------------------
 
+// (vs_lds: the per-channel V scales of this (batch, head) in LDS instead of a.vscale in global memory.)
 template <int DT, int D, int PV>
-__global__ void __launch_bounds__(256) prep_v_kernel(PrepVArgs a) {
+__device__ __forceinline__ void prep_v_tile(const PrepVArgs& a, const int pidx, const int h, const int b, const float* vs_lds) {
   // A lane converts 4 consecutive rows x 8 consecutive channels at a time, so that the 4 row values of
   // a channel pack into one dword (fp8) or two (fp16): exactly the (b = 0..3) group of the panel
   // order.  They are staged in LDS as T[channel][row quad] and read back in panel order.
@@ -279,7 +289,6 @@ __global__ void __launch_bounds__(256) prep_v_kernel(PrepVArgs a) {
   constexpr int PANEL_BYTES = kPanelRows * D * ESZ;
   constexpr int DTN = D / 32;
   __shared__ uint32_t T[D * TS];
-  const int pidx = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
   const int tid = threadIdx.x, tr = tid / TPR, tc = tid % TPR;
   int L = a.L;
   int64_t vbase, pbase;
@@ -299,7 +308,7 @@ __global__ void __launch_bounds__(256) prep_v_kernel(PrepVArgs a) {
   if constexpr (PV == 1) {
 #pragma unroll
     for (int i = 0; i < 8; i++) {
-      sc[i] = a.vscale[((int64_t)b * a.H + h) * D + tc * 8 + i];
+      sc[i] = vs_lds ? vs_lds[tc * 8 + i] : a.vscale[((int64_t)b * a.H + h) * D + tc * 8 + i];
       rc[i] = 1.0f / sc[i];
       fast = fast && ((__builtin_bit_cast(uint32_t, sc[i]) & 0x7fffffu) != 0x7fffffu) && sc[i] < 1.0e30f;
     }
@@ -359,6 +368,96 @@ __global__ void __launch_bounds__(256) prep_v_kernel(PrepVArgs a) {
   }
 }
 
+template <int DT, int D, int PV>
+__global__ void __launch_bounds__(256) prep_v_kernel(PrepVArgs a) {
+  prep_v_tile<DT, D, PV>(a, blockIdx.x, blockIdx.y, blockIdx.z, nullptr);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Short sequences: every pre-pass of the one-call pipeline in ONE launch.  A workgroup is either a K tile or a V panel
+// of one (batch, kv-head); it first computes the statistic its tile needs over the whole sequence itself (the K mean:
+// float64 sums in the order of the two-stage kernels above -- per 512-row chunk, per-lane rows, the lanes of a channel
+// in order, chunks in order -- so that the mean is the same bit pattern; the V scale: an abs-max, which has no order)
+// and then runs the tile code of the kernels above.  The statistics are read again by every workgroup of the
+// (batch, head): affordable while the sequence is short and the reads hit the L2; six dependent launches of a few
+// microseconds each become one.
+// ---------------------------------------------------------------------------------------------
+template <int DT, int D, int PV>
+__global__ void __launch_bounds__(256) prepass_small_kernel(QuantArgs qa, PrepVArgs va, int nk, int smooth, u16* km_out,
+                                                            float* vscale_out) {
+  constexpr int TPR = D / 8, RPP = 256 / TPR;
+  const int h = blockIdx.y, b = blockIdx.z;
+  const int tid = threadIdx.x, tr = tid / TPR, tc = tid % TPR;
+  __shared__ double red[RPP][D];
+  __shared__ u16 km_l[D];
+  __shared__ float vs_l[D];
+  if ((int)blockIdx.x < nk) {
+    if (smooth) {
+      const int L = qa.L;
+      const int64_t xbase = (int64_t)b * qa.x_sb + (int64_t)h * qa.x_sh;
+      double s = 0;
+      for (int n0 = 0; n0 < L; n0 += kChunkRows) {
+        const int n1 = min(L, n0 + kChunkRows);
+        double acc[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) acc[i] = 0;
+#pragma unroll 8
+        for (int n = n0 + tr; n < n1; n += RPP) {   // (unrolled for loads in flight; the additions keep their order)
+          uint4 raw = *reinterpret_cast<const uint4*>(qa.x + xbase + (int64_t)n * qa.x_sn + tc * 8);
+          const u16* e = reinterpret_cast<const u16*>(&raw);
+#pragma unroll
+          for (int i = 0; i < 8; i++) acc[i] += (double)to_f32<DT>(e[i]);
+        }
+#pragma unroll
+        for (int i = 0; i < 8; i++) red[tr][tc * 8 + i] = acc[i];
+        __syncthreads();
+        if (tid < D) {
+          double t = red[0][tid];
+          for (int r = 1; r < RPP; r++) t += red[r][tid];
+          s += t;
+        }
+        __syncthreads();
+      }
+      if (tid < D) {
+        const u16 m = from_f32<DT>(L > 0 ? (float)(s / (double)L) : 0.f);
+        km_l[tid] = m;
+        if (blockIdx.x == 0) km_out[((int64_t)b * qa.H + h) * D + tid] = m;
+      }
+      __syncthreads();
+    }
+    quant_int8_tile<DT, D>(qa, blockIdx.x, h, b, smooth ? km_l : nullptr);
+  } else {
+    const int pidx = blockIdx.x - nk;
+    if constexpr (PV == 1) {
+      const int L = va.L;
+      const int64_t vbase = (int64_t)b * va.v_sb + (int64_t)h * va.v_sh;
+      float acc[8];
+#pragma unroll
+      for (int i = 0; i < 8; i++) acc[i] = 0.f;
+#pragma unroll 8
+      for (int n = tr; n < L; n += RPP) {
+        uint4 raw = *reinterpret_cast<const uint4*>(va.v + vbase + (int64_t)n * va.v_sn + tc * 8);
+        const u16* e = reinterpret_cast<const u16*>(&raw);
+#pragma unroll
+        for (int i = 0; i < 8; i++) acc[i] = fmaxf(acc[i], fabsf(to_f32<DT>(e[i])));
+      }
+      float* redf = reinterpret_cast<float*>(&red[0][0]);
+#pragma unroll
+      for (int i = 0; i < 8; i++) redf[tr * D + tc * 8 + i] = acc[i];
+      __syncthreads();
+      if (tid < D) {
+        float t = redf[tid];
+        for (int r = 1; r < RPP; r++) t = fmaxf(t, redf[r * D + tid]);
+        const float sc = fmaxf(t / 448.0f, kScaleFloor);
+        vs_l[tid] = sc;
+        if (pidx == 0) vscale_out[((int64_t)b * va.H + h) * D + tid] = sc;
+      }
+      __syncthreads();
+    }
+    prep_v_tile<DT, D, PV>(va, pidx, h, b, PV == 1 ? vs_l : nullptr);
+  }
+}
+
 // ---------------------------------------------------------------------------------------------
 // Host-side launchers (called from the C ABI in sage_api.hip).
 // ---------------------------------------------------------------------------------------------
@@ -399,6 +498,22 @@ hipError_t launch_v_scale(const ColStatArgs& a, int dtype, float* vscale, hipStr
   if (e != hipSuccess) return e;
   dim3 grid(a.H, a.B), block(a.D);
   vscale_finalize_kernel<<<grid, block, 0, st>>>((const float*)a.partial, vscale, a.H, a.L, a.D, a.nchunk, a.cu_seqlens);
+  return hipGetLastError();
+}
+
+hipError_t launch_prepass_small(const QuantArgs& qa, const PrepVArgs& va, int dtype, int pv, int nk, int nv, int smooth,
+                                void* km_out, float* vscale_out, hipStream_t st) {
+  if (nk + nv == 0 || qa.B == 0 || qa.H == 0) return hipSuccess;
+  dim3 grid(nk + nv, qa.H, qa.B), block(256);
+#define SAGE_PREPASS(DT, DD, PVV) prepass_small_kernel<DT, DD, PVV><<<grid, block, 0, st>>>(qa, va, nk, smooth, (u16*)km_out, vscale_out)
+  if (dtype == 0) {
+    if (qa.D == 64) { if (pv) SAGE_PREPASS(0, 64, 1); else SAGE_PREPASS(0, 64, 0); }
+    else { if (pv) SAGE_PREPASS(0, 128, 1); else SAGE_PREPASS(0, 128, 0); }
+  } else {
+    if (qa.D == 64) { if (pv) SAGE_PREPASS(1, 64, 1); else SAGE_PREPASS(1, 64, 0); }
+    else { if (pv) SAGE_PREPASS(1, 128, 1); else SAGE_PREPASS(1, 128, 0); }
+  }
+#undef SAGE_PREPASS
   return hipGetLastError();
 }
 

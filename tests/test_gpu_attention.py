@@ -218,6 +218,37 @@ def test_lse_is_empty_unless_requested():
     assert lse.numel() == 0 and out.dtype == torch.float16
 
 
+@pytest.mark.parametrize("smooth", [True, False])
+@pytest.mark.parametrize("pv", ["fp16", "fp8"])
+@pytest.mark.parametrize("cfg", [("HND", 1, 8, 8, 1024, 1024, 64, torch.float16, 128, 128),      # BASELINE config 0's shape
+                                 ("NHD", 2, 4, 2, 300, 1000, 128, torch.bfloat16, 64, 64),
+                                 ("HND", 1, 2, 1, 129, 1024, 128, torch.bfloat16, 32, 16),
+                                 ("HND", 1, 2, 1, 40, 1025, 128, torch.bfloat16, 64, 128),     # one key too many: the six-launch path
+                                 ("HND", 3, 2, 2, 77, 513, 64, torch.float16, 128, 32)])
+def test_one_call_on_short_sequences_equals_the_separate_calls_bitwise(cfg, pv, smooth):
+    """Up to 1024 keys (and 4 M elements of K) the one-call pipeline runs its K and V pre-passes as ONE launch, whose workgroups compute the K
+    mean / V scale of their sequence themselves; the separate entry points use the two-stage statistics kernels.  Same
+    int8 K, same scales, same panels: the attention output (and the LSE, which also sees the K mean) must be the same
+    bits.  Sequence lengths off every block size, GQA, both layouts, the largest length of the short path and the first
+    beyond it."""
+    layout, B, Hq, Hkv, Sq, Skv, D, dtype, blkq, blkk = cfg
+    g = torch.Generator().manual_seed(31 + Sq + Skv)
+    q = randn(layout, B, Hq, Sq, D, dtype, g).to(DEV)
+    k = (randn(layout, B, Hkv, Skv, D, dtype, g) + 0.5).to(DEV)     # a mean worth removing
+    v = randn(layout, B, Hkv, Skv, D, dtype, g).to(DEV)
+    one, lse1 = sa.sageattn(q, k, v, tensor_layout=layout, smooth_k=smooth, pv_mode=pv, BLKQ=blkq, BLKK=blkk, return_lse=True)
+    one_plain = sa.sageattn(q, k, v, tensor_layout=layout, smooth_k=smooth, pv_mode=pv, BLKQ=blkq, BLKK=blkk)
+    km = sa.k_mean(k, layout) if smooth else None
+    _, _, ki, ks = sa.per_block_int8(q, k, km=km, BLKQ=blkq, BLKK=blkk, tensor_layout=layout)
+    sep, _ = sa.forward_fused_q(q, ki, v, ks, tensor_layout=layout, output_dtype=dtype, BLKQ=blkq, BLKK=blkk, pv_mode=pv)
+    assert torch.equal(one_plain, sep)
+    # the LSE variant runs the standalone Q pass; its output against the same pass made by hand
+    qi, qs, _, _ = sa.per_block_int8(q, k, km=km, BLKQ=blkq, BLKK=blkk, tensor_layout=layout)
+    sep2, _ = sa.forward(qi, ki, v, qs, ks, tensor_layout=layout, output_dtype=dtype, BLKQ=blkq, BLKK=blkk, pv_mode=pv,
+                         return_lse=True)
+    assert torch.equal(one, sep2) and torch.isfinite(lse1).all()
+
+
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("shape", [(1, 2, 1, 129, 70), (2, 4, 2, 300, 1000), (1, 3, 3, 513, 513)])
 @pytest.mark.parametrize("D", [64, 128])
