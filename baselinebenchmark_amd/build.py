@@ -25,6 +25,13 @@ FLAGS = [
 ]
 
 
+# The instantiation units of the shipped attention kernels are scheduled for instruction-level parallelism rather than
+# for occupancy (which is fixed at two wavefronts per SIMD anyway): +0.9 % on config 2 and on FP16 P.V at 16k keys, equal
+# elsewhere, no scratch.  The explicit-mask variants (sage_attn_mask.hip), which spill under either strategy, keep the default.
+EXTRA_FLAGS = {src: ["-mllvm", "-amdgpu-sched-strategy=max-ilp"]
+               for src in ("sage_attn.hip", "sage_attn_qfuse.hip", "sage_attn_kinterleave.hip")}
+
+
 def _hipcc() -> str:
     return os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
@@ -34,7 +41,7 @@ TIMING_LIB = CSRC / "libsage_mi355x_timing.so"   # same library with in-kernel i
 
 def _compile(src: str, timing: bool = False) -> Path:
     obj = CSRC / (src.replace(".hip", ".timing.o" if timing else ".o"))
-    cmd = [_hipcc(), *FLAGS, *(["-DSAGE_TIMING=1"] if timing else []), "-c", str(CSRC / src), "-o", str(obj)]
+    cmd = [_hipcc(), *FLAGS, *EXTRA_FLAGS.get(src, []), *(["-DSAGE_TIMING=1"] if timing else []), "-c", str(CSRC / src), "-o", str(obj)]
     res = subprocess.run(cmd, capture_output=True, text=True)
     noise = "is not a recognized feature for this target"
     err = "\n".join(l for l in res.stderr.splitlines() if noise not in l)
