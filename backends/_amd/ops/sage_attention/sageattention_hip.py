@@ -2,7 +2,8 @@
 
 The names, arguments and error behaviour are those of the other vendors' interface files
 (backends/_hygon/ops/sageattention/sageattention_hip.py:37-80 for ``per_block_int8`` / ``forward`` /
-``backend_name``; backends/_enflame/ops/sage_attention/core.py for ``sageattn`` / ``sageattn_varlen``).  The work is
+``backend_name``; backends/_metax/ops/sage_attention/official_wheel.py:18-24 for ``sageattn``, whose packed counterpart
+here is ``sageattn_varlen``).  The work is
 done by the HIP library behind the ``baselinebenchmark_amd`` package; this file adds nothing to it.  There is no
 fallback: importing this file without the built library raises.
 """

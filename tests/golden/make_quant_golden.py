@@ -13,6 +13,8 @@ import os
 import sys
 
 os.environ.setdefault("TRITON_INTERPRET", "1")
+os.environ.setdefault("PYTHONDONTWRITEBYTECODE", "1")
+sys.dont_write_bytecode = True   # importing the reference must not write a __pycache__ into its (read-only) tree
 
 import numpy as np
 import torch

@@ -122,6 +122,28 @@ def test_k_mean_and_smoothed_quantisation(layout, dtype):
     _cmp(q, k, km=km_ref, layout=layout)
 
 
+@pytest.mark.parametrize("dtype,precision", [(torch.float16, 11), (torch.bfloat16, 8)])
+@pytest.mark.parametrize("L", [128, 1300])
+def test_k_mean_rounding_order_on_tie_channels(dtype, precision, L):
+    # channels whose exact mean sits a hair above a half-way point of the dtype (tests/test_oracle_quant.py pins the oracle's
+    # value for them with exact rationals): a float32 accumulation or a single rounding would give another value
+    g = torch.Generator().manual_seed(33)
+    k = randn("HND", 1, 2, L, 64, dtype, g, offset_std=2.0)
+    h = 2.0 ** -precision
+    col0 = torch.full((L,), 2.0 ** -18)
+    col0[0], col0[1], col0[2] = L / 2, L / 2, L * h
+    col1 = torch.zeros(L)
+    col1[0], col1[1], col1[2], col1[3] = L / 2, L / 2, L * h, 2.0 ** -24
+    if L == 128:
+        k[0, 0, :, 0], k[0, 0, :, 1] = col0.to(dtype), col1.to(dtype)
+    else:   # the same values spread over the two-stage reduction's 512-row chunks (last first)
+        k[0, 0, :, 0], k[0, 0, :, 1] = col0.flip(0).to(dtype), col1.flip(0).to(dtype)
+    km = sa.k_mean(k.to(DEV), "HND").cpu()
+    assert torch.equal(km, oq.k_mean(k, "HND"))
+    if L == 128:
+        assert float(km[0, 0, 0, 0]) == 1.0 + 2 * h and float(km[0, 0, 0, 1]) == 1.0
+
+
 def test_adversarial_values():
     # ties at .5, +-max, zeros, a zero tile, tiny values below the scale floor and huge magnitudes
     g = torch.Generator().manual_seed(33)

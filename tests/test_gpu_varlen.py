@@ -107,7 +107,9 @@ def test_random_packed_batches_match_sdpa_and_the_fixed_length_call(c):
     for i in range(len(c["lens"])):
         a, b = int(cu[i]), int(cu[i + 1])
         m = oa.metrics(out[a:b].cpu().float(), ref[a:b])
-        assert m["finite"] and m["cosine"] >= 0.998, (i, c["lens"][i], m)
+        # the north-star gate; sequences of a few rows get a stated looser one (a cosine over one or two rows of D numbers
+        # is dominated by the e4m3 rounding of a handful of probabilities that nothing averages)
+        assert m["finite"] and m["cosine"] >= (0.999 if c["lens"][i] >= 64 else 0.995), (i, c["lens"][i], m)
         one = sa.sageattn(qd[a:b].unsqueeze(0), kd[a:b].unsqueeze(0), vd[a:b].unsqueeze(0), tensor_layout="NHD", **kw)
         assert torch.equal(one[0], out[a:b]), (i, c["lens"][i])
 

@@ -153,12 +153,70 @@ def test_exhaustive_fp16_values_single_tile():
 
 
 def test_k_mean_definition():
+    # The reference never computes km (it is an argument of per_block_int8), so this is a DEFINITION, not parity: the
+    # bound below catches a wrong axis or a missing division, the exact-rational test after it fixes the rounding order.
     g = torch.Generator().manual_seed(5)
     k = randn("NHD", 2, 3, 333, 64, torch.bfloat16, g, offset_std=2.0)
     km = oq.k_mean(k, "NHD")
     assert km.shape == (2, 1, 3, 64) and km.dtype == torch.bfloat16
     ref = k.double().mean(dim=1, keepdim=True)
     assert torch.all((km.double() - ref).abs() <= ref.abs() * 2 ** -8 + 1e-30)
+
+
+def _round_fraction(x, precision, emin):
+    """Round-to-nearest-even of an exact rational to a binary float with `precision` significand bits and minimum
+    normal exponent `emin` (subnormals below it), returned as an exact Fraction."""
+    from fractions import Fraction
+    if x == 0:
+        return Fraction(0)
+    sign, a = (-1 if x < 0 else 1), abs(x)
+    e = a.numerator.bit_length() - a.denominator.bit_length()
+    if Fraction(2) ** e > a:
+        e -= 1                                   # now 2^e <= a < 2^(e+1)
+    ulp = Fraction(2) ** (max(e, emin) - (precision - 1))
+    n = a / ulp
+    lo = n.numerator // n.denominator
+    rem = n - lo
+    if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and lo % 2 == 1):
+        lo += 1
+    return sign * lo * ulp
+
+
+@pytest.mark.parametrize("dtype,precision,emin", [(torch.float16, 11, -14), (torch.bfloat16, 8, -126)])
+def test_k_mean_against_exact_rational_arithmetic(dtype, precision, emin):
+    # Definition: mean = exact sum / L, rounded ONCE to binary32 and then once to the input dtype.  Two channels are built
+    # so that a plausible other order gives another value (checked at the end), which pins the rounding order and not
+    # only the axis:
+    #   channel 0: 64 + 64 + 128*h + 125 values of 2^-18 (h = half a step of the dtype at 1.0).  The exact mean lies just
+    #     above the half-way point 1 + h and rounds up; a float32 accumulation along the sequence drops every 2^-18
+    #     (half an ulp of 128.x is 2^-17), lands on the tie and rounds to even, 1.0.
+    #   channel 1: 2 + 2 + 4*h + 2^-38 + zeros ... over L = 4 would do; with L = 128: 64 + 64 + 128*h + 2^-24.  The exact
+    #     mean is the half-way point plus 2^-31: binary32 rounds it to the tie, which then goes to even (1.0); rounding
+    #     the exact mean directly to the dtype goes up.
+    from fractions import Fraction
+    g = torch.Generator().manual_seed(11)
+    L, C = 128, 12
+    h = 2.0 ** -precision
+    k = (torch.randn((1, 1, L, C), generator=g) * 3.0 + torch.randn((1, 1, 1, C), generator=g) * 40.0).to(dtype)
+    col0 = torch.full((L,), 2.0 ** -18)
+    col0[0], col0[1], col0[2] = 64.0, 64.0, 128 * h
+    col1 = torch.zeros(L)
+    col1[0], col1[1], col1[2], col1[3] = 64.0, 64.0, 128 * h, 2.0 ** -24
+    k[0, 0, :, 0], k[0, 0, :, 1] = col0.to(dtype), col1.to(dtype)
+    assert torch.equal(k[0, 0, :, 0].double(), col0.double()) and torch.equal(k[0, 0, :, 1].double(), col1.double())
+    km = oq.k_mean(k, "HND")
+    for c in range(C):
+        total = sum(Fraction(float(k[0, 0, n, c])) for n in range(L))       # fp16/bf16 values are exact Fractions
+        want = _round_fraction(_round_fraction(total / L, 24, -126), precision, emin)
+        assert Fraction(float(km[0, 0, 0, c])) == want, (c, float(km[0, 0, 0, c]), float(want))
+    assert float(km[0, 0, 0, 0]) == 1.0 + 2 * h and float(km[0, 0, 0, 1]) == 1.0
+    # the other orders, on the same tensor
+    acc = torch.zeros((), dtype=torch.float32)
+    for n in range(L):
+        acc = acc + k[0, 0, n, 0].float()
+    assert float((acc / L).to(dtype)) == 1.0                                               # float32 accumulation: the tie
+    total1 = sum(Fraction(float(k[0, 0, n, 1])) for n in range(L))
+    assert _round_fraction(total1 / L, precision, emin) == Fraction(1) + Fraction(2) * Fraction(h)   # one rounding: up
 
 
 def test_fp8_value_set_matches_reference_bit_decoder():
