@@ -285,6 +285,7 @@ int attn_impl(const int8_t* q, const int8_t* k, const void* v_panels, const floa
     grid = (int64_t)a.nqt * B * Hq;
   }
   if (grid > 0x7fffffff) return fail(SAGE_EINVAL, "too many tiles for one launch");
+  finish_attn_args(a, is_causal != 0);
   hipError_t e = launch_attn(a, D, pv_mode, is_causal != 0, (int)grid, (hipStream_t)stream);
   if (e != hipSuccess) return hip_fail(e, "sage_attn_fwd");
   return SAGE_OK;

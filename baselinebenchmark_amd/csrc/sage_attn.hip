@@ -127,6 +127,29 @@ AttnConfig attn_config(int D, int pv, bool packed) {
   return c;
 }
 
+void finish_attn_args(AttnArgs& a, bool causal) {
+  const bool packed = a.cu_q != nullptr;
+  a.G = a.Hq / a.Hkv;
+  const int heads = packed ? a.Hq : a.B * a.Hq, groups = packed ? a.Hkv : a.B * a.Hkv;
+  a.div_G = make_fastdiv(a.G);
+  a.div_Hkv = make_fastdiv(a.Hkv);
+  a.div_heads = make_fastdiv(heads > 0 ? heads : 1);
+  a.tier_shift = -1;
+  a.div_range = a.div_last = make_fastdiv(1);
+  // Per-XCD tile order (fixed-length batches whose heads and KV groups spread evenly over the eight XCDs): ranges of
+  // R = 2^tier_shift consecutive q-tiles, R at most 32 and at most half of a head's q-tiles.  Causal problems with fewer than
+  // 16 q-tiles per compute unit keep the plain heaviest-first order: with so few rounds the balance of the last one
+  // matters more than locality (5 % on 4 x 32 heads of 4096 rows).
+  if (!packed && (heads & 7) == 0 && (groups & 7) == 0 && (!causal || (int64_t)a.nqt * (heads >> 3) >= 512)) {
+    int shift = 5;
+    while (shift > 0 && (2 << shift) > a.nqt) shift--;
+    a.tier_shift = shift;
+    const int R = 1 << shift, hpx = heads >> 3, last = a.nqt - (a.nqt >> shift << shift);
+    a.div_range = make_fastdiv((uint32_t)R * hpx);
+    a.div_last = make_fastdiv(last > 0 ? last : 1);
+  }
+}
+
 hipError_t launch_attn(const AttnArgs& a, int D, int pv, bool causal, int grid, hipStream_t st) {
   if (grid == 0) return hipSuccess;
   if (a.mask) return launch_attn_masked(a, D, pv, grid, st);
@@ -136,9 +159,12 @@ hipError_t launch_attn(const AttnArgs& a, int D, int pv, bool causal, int grid, 
   // Row sums on the matrix pipe unless LSE is wanted (FP16 P.V: only head_dim 64 gains by it; head_dim 128 is
   // bound by its matrix phases and keeps the sums on the vector ALU).
   const bool msum = a.lse == nullptr;
-#define SAGE_ATTN(DD, PVV, BNN, MS) (causal ? launch_one<DD, 8, BNN, PVV, true, MS, 0>(a, grid, st) : launch_one<DD, 8, BNN, PVV, false, MS, 0>(a, grid, st))
+  // (K scale blocks of 64 / 128 keys: the variants that know which 32-key groups share a scale)
+#define SAGE_ATTN_W(DD, PVV, BNN, MS, KWW) (causal ? launch_one<DD, 8, BNN, PVV, true, MS, 0, 1, false, KWW>(a, grid, st) : launch_one<DD, 8, BNN, PVV, false, MS, 0, 1, false, KWW>(a, grid, st))
+#define SAGE_ATTN(DD, PVV, BNN, MS) (a.blkk >= 128 ? SAGE_ATTN_W(DD, PVV, BNN, MS, 4) : a.blkk == 64 ? SAGE_ATTN_W(DD, PVV, BNN, MS, 2) : SAGE_ATTN_W(DD, PVV, BNN, MS, 1))
   if (D == 128) return pv ? (msum ? SAGE_ATTN(128, 1, 128, true) : SAGE_ATTN(128, 1, 128, false)) : SAGE_ATTN(128, 0, 128, false);
   return pv ? (msum ? SAGE_ATTN(64, 1, 128, true) : SAGE_ATTN(64, 1, 128, false)) : (msum ? SAGE_ATTN(64, 0, 128, true) : SAGE_ATTN(64, 0, 128, false));
+#undef SAGE_ATTN_W
 #undef SAGE_ATTN
 }
 

@@ -53,6 +53,10 @@ constexpr float kCodeBias = -0.3f;       // centres the linear-mantissa fp8 code
 template <int PV> struct PCfg;
 template <> struct PCfg<1> { static constexpr float tau = 3.0f, pshift = 5.0f; };   // fp8: p*32 <= 256 < 448
 template <> struct PCfg<0> { static constexpr float tau = 8.0f, pshift = 0.0f; };   // fp16: p <= 256
+// Block-scaled probability codes (FP8 P.V kernels without LSE or an explicit mask, see softmax): the largest probability of a
+// query row in a 128-key tile is coded within one binade below 2^kBlockTop (code <= 126 = 448), the block's power-of-two
+// scale goes to the MFMA as an E8M0 byte, kBlockScaleBias + exponent; the running maximum then only has to keep fp32 in range.
+constexpr float kBlockTop = 8.75f, kBlockTau = 20.0f, kBlockMinExp = -110.0f, kBlockScaleBias = 119.0f;   // 119 = 127 - 8
 
 // NOTE: __builtin_bit_cast applied directly to an element of an ext_vector_type value reads element
 // 0 whatever the index (clang miscompiles the element lvalue), so vector elements are always passed
@@ -143,7 +147,10 @@ static __device__ unsigned long long g_tile_timing[kTimingSets][48];
 // KSUB: K scale blocks per 32 keys (1 for blocks of 32/64/128 keys, 2 for blocks of 16 keys); 3 = four interleaved scales per
 // block of 32/64/128 keys, scale t for the keys n of the block with (n % 8) / 2 == t (two of them reach every lane).
 // QF: the kernel reads fp16/bf16 Q and quantises its own tile (same arithmetic as quant_int8_kernel).
-template <int D, int NW, int BN, int PV, bool CAUSAL, bool MSUM, int MASK, int KSUB = 1, bool QF = false>
+// KW (with KSUB == 1): 32-key groups that are known to share a K scale -- 1 for any block size from 32 keys on (every group
+// looks its scale up), 2 for blocks of 64 keys and more, 4 for blocks of 128: the row maximum then runs one integer chain
+// per scale and the per-scale constants of the softmax are computed once (a tenth of the vector instructions of a tile).
+template <int D, int NW, int BN, int PV, bool CAUSAL, bool MSUM, int MASK, int KSUB = 1, bool QF = false, int KW = 1>
 __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
   constexpr int GSH = SAGE_GSH;   // which bit of the wavefront index picks the group
   static_assert(NW == (2 << GSH), "the two groups pair wavefront w with w + NW/2");
@@ -183,16 +190,17 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
   const int m = lane & 31, h = lane >> 5;
 
   // ---- which tile am I: heaviest q-tiles first; q-heads sharing a KV head on one XCD ----
+  // (Divisions by launch constants go through host-made multipliers, range widths are powers of two: every workgroup
+  // pays for this decode before its first memory request.)
   const bool packed = a.cu_q != nullptr;
-  const int G = a.Hq / a.Hkv;
+  const int G = a.G;
+  const uint32_t bid = blockIdx.x;
   int rank, s, NG;
-  if (packed) { rank = blockIdx.x / a.Hq; s = blockIdx.x % a.Hq; NG = a.Hkv; }
+  if (packed) { rank = fastdiv(bid, a.div_heads); s = bid - rank * a.Hq; NG = a.Hkv; }
   else {
     const int U = a.B * a.Hq;
     NG = a.B * a.Hkv;
-    // (Causal problems with fewer than 16 q-tiles per compute unit keep the plain heaviest-first order: with so few
-    // rounds the balance of the last one matters more than locality -- 5 % on 4 x 32 heads of 4096 rows.)
-    if ((U & 7) == 0 && (NG & 7) == 0 && (!CAUSAL || a.nqt * (U >> 3) >= 512)) {
+    if (a.tier_shift >= 0) {
       // Inside an XCD (workgroup index modulo 8; 32 compute units) the workgroups that run at the same time take
       // neighbouring q-tiles of FEW heads: the q-tiles of a head (by weight: rank 0 is the heaviest) are cut into ranges
       // of R consecutive ranks, and the XCD goes through a range head by head, a head's R q-tiles in a row, before it
@@ -201,40 +209,43 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
       // of a head walk the same K/V tiles from tile 0 on at about the same pace, so one of them fetches a tile into the
       // XCD's L2 and the others hit it there (a quarter of the L2 fills of the plain heaviest-first order, where an XCD
       // works on all its heads at once), and neighbouring q-tiles read neighbouring rows of Q.
-      const int x = blockIdx.x & 7, hpx = U >> 3;   // XCD, heads per XCD
-      int l = blockIdx.x >> 3;                      // index inside the XCD
-      int R = 32;
-      while (R > 1 && 2 * R > a.nqt) R >>= 1;
+      const int x = bid & 7, hpx = U >> 3;   // XCD, heads per XCD
+      int l = bid >> 3;                      // index inside the XCD
+      int rs = a.tier_shift;                 // log2 of the range width R
       if constexpr (CAUSAL) {
         // Causal q-tiles get lighter with their rank, and the ranges narrower: never more than half of the ranks that
         // are left (64 q-tiles: 32, 16, 8, 4, 2, 1, 1), so that the workgroups an XCD runs last are all short ones
         // (+2.5 % on 64 x 32 heads of 1024 rows, nothing on long sequences).
         int r0 = 0;
         for (;;) {
-          while (R > 1 && 2 * R > a.nqt - r0) R >>= 1;
-          if (l < R * hpx) break;
-          l -= R * hpx;
-          r0 += R;
+          while (rs > 0 && (2 << rs) > a.nqt - r0) rs--;
+          if (l < (hpx << rs)) break;
+          l -= hpx << rs;
+          r0 += 1 << rs;
           if (r0 >= a.nqt) return;   // (a grid larger than the tile count: nothing to do)
         }
-        rank = r0 + l % R;
-        s = x + 8 * (l / R);
+        rank = r0 + (l & ((1 << rs) - 1));
+        s = x + 8 * (l >> rs);
       } else {
         // all q-tiles cost the same: ranges of R ranks and one last range with the remainder
-        const int nfull = a.nqt / R, lfull = nfull * R * hpx;
-        int t, Rt, lr;                              // range, its width, index inside it
-        if (l < lfull) { t = l / (R * hpx); Rt = R; lr = l % (R * hpx); }
-        else { t = nfull; Rt = a.nqt - nfull * R; lr = l - lfull; }
-        rank = t * R + lr % Rt;
-        s = x + 8 * (lr / Rt);
+        const int nfull = a.nqt >> rs, lfull = (nfull * hpx) << rs;
+        if (l < lfull) {
+          const int t = fastdiv(l, a.div_range), lr = l - ((t * hpx) << rs);
+          rank = (t << rs) + (lr & ((1 << rs) - 1));
+          s = x + 8 * (lr >> rs);
+        } else {
+          const int Rt = a.nqt - (nfull << rs), lr = l - lfull, hd = fastdiv(lr, a.div_last);
+          rank = (nfull << rs) + lr - hd * Rt;
+          s = x + 8 * hd;
+        }
       }
     } else {
-      rank = blockIdx.x / U; s = blockIdx.x % U;
+      rank = fastdiv(bid, a.div_heads); s = bid - rank * U;
     }
   }
   int gi, g;
-  if ((NG & 7) == 0) { int x = s & 7, y = s >> 3; gi = x + 8 * (y / G); g = y % G; }
-  else { gi = s / G; g = s % G; }
+  if ((NG & 7) == 0) { const int x = s & 7, y = s >> 3, yg = fastdiv(y, a.div_G); gi = x + 8 * yg; g = y - yg * G; }
+  else { gi = fastdiv(s, a.div_G); g = s - gi * G; }
   int b, kvh, qt, Lq, Lk, hq_idx;
   int64_t qoff, koff, ooff, lseoff;
   const float *qsp, *ksp;
@@ -256,7 +267,7 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
     ksp = a.ks + (int64_t)kvh * a.ks_sh + a.cu_kblk[b];
     vbase = a.vp + ((int64_t)kvh * a.panel_sh + a.cu_panel[b]) * PANEL_BYTES;
   } else {
-    b = gi / a.Hkv; kvh = gi % a.Hkv;
+    b = fastdiv(gi, a.div_Hkv); kvh = gi - b * a.Hkv;
     qt = CAUSAL ? a.nqt - 1 - rank : rank;
     Lq = a.Sq; Lk = a.Skv;
     int hq = kvh * G + g;
@@ -265,11 +276,11 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
     ooff = (int64_t)b * a.o_sb + (int64_t)hq * a.o_sh;
     koff = (int64_t)b * a.k_sb + (int64_t)kvh * a.k_sh;
     lseoff = ((int64_t)b * a.Hq + hq) * a.Sq;
-    qsp = a.qs + (((int64_t)b * a.Hq + hq) * ((Lq + a.blkq - 1) / a.blkq) << a.qg_shift);
-    ksp = a.ks + ((int64_t)b * a.Hkv + kvh) * ((Lk + a.blkk - 1) / a.blkk) * (KSUB == 3 ? 4 : 1);
+    qsp = a.qs + (((int64_t)b * a.Hq + hq) * ((Lq + a.blkq - 1) >> a.blkq_shift) << a.qg_shift);
+    ksp = a.ks + ((int64_t)b * a.Hkv + kvh) * ((Lk + a.blkk - 1) >> a.blkk_shift) * (KSUB == 3 ? 4 : 1);
     vbase = a.vp + ((int64_t)b * a.Hkv + kvh) * ((Lk + kPanelRows - 1) / kPanelRows) * PANEL_BYTES;
   }
-  nkblk = (Lk + a.blkk - 1) / a.blkk;
+  nkblk = (Lk + a.blkk - 1) >> a.blkk_shift;
   // The K scales are read through the scalar cache (constant address space): a vector load would sit
   // in the same in-order counter as the tile loads in flight and make every tile wait for them.
   const __attribute__((address_space(4))) float* ksc = (const __attribute__((address_space(4))) float*)ksp;
@@ -333,21 +344,49 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
     for (int i = 0; i < VPIECES; i++) dma16(vrsrc, voffv[i], j * VBYTES + dw * 1024, dst + (i * NW + wl) * 1024);
   };
 
-  // The first K tile is requested before anything else waits on memory, and the per-channel V scales
-  // of the epilogue come along (4 bytes per lane, D / 64 wavefronts).
-  if (ntiles > 0) load_k(0, dw_self);
+  // The K tiles of the lead are requested before anything waits on memory, and the per-channel V scales of the epilogue
+  // come along (4 bytes per lane, D / 64 wavefronts).  Kernels that quantise their own Q put the raw q-tile's requests in
+  // front of these (the quantisation is what the prologue waits for; the K tiles then arrive under it).
   float* vs_lds = reinterpret_cast<float*>(smem + attn_tile_lds_bytes<D, NW, BN, PV, CAUSAL, QF>());
-  if constexpr (PV == 1) {
-    if (w < D / 64) {
-      if (Lk > 0) {
-        const __amdgpu_buffer_rsrc_t vsrsrc =
-            __builtin_amdgcn_make_buffer_rsrc((void*)(a.vs + ((int64_t)b * a.Hkv + kvh) * D), 0, D * 4, 0x00020000);
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(vsrsrc, (__attribute__((address_space(3))) void*)(vs_lds + 64 * w), 4, lane * 4, w * 256, 0, 0);
-      } else {
-        vs_lds[64 * w + lane] = 1.0f;   // no keys: nothing ever wrote the scales, and 0 * garbage must stay 0
+  // returns the number of requests this wavefront issued
+  auto request_lead_tiles = [&]() -> int {
+    int n = 0;
+    if (ntiles > 0) { load_k(0, dw_self); n += KPIECES; }
+    if constexpr (PV == 1) {
+      if (w < D / 64) {
+        if (Lk > 0) {
+          const __amdgpu_buffer_rsrc_t vsrsrc =
+              __builtin_amdgcn_make_buffer_rsrc((void*)(a.vs + ((int64_t)b * a.Hkv + kvh) * D), 0, D * 4, 0x00020000);
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(vsrsrc, (__attribute__((address_space(3))) void*)(vs_lds + 64 * w), 4, lane * 4, w * 256, 0, 0);
+          n += 1;
+        } else {
+          vs_lds[64 * w + lane] = 1.0f;   // no keys: nothing ever wrote the scales, and 0 * garbage must stay 0
+        }
       }
     }
-  }
+#pragma unroll
+    for (int t = 1; t < LEAD; t++)
+      if (t < ntiles) { load_k(t, dw_self); n += KPIECES; }
+    return n;
+  };
+  // Tile loads complete in the order they were requested, so waiting until only the n newest are in
+  // flight leaves exactly the n last requests outstanding.
+  auto wait_all_but = [&](int n) {
+    switch (n) {
+      case 0: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+      case 1: asm volatile("s_waitcnt vmcnt(1)" ::: "memory"); break;
+      case 2: asm volatile("s_waitcnt vmcnt(2)" ::: "memory"); break;
+      case 3: asm volatile("s_waitcnt vmcnt(3)" ::: "memory"); break;
+      case 4: asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); break;
+      case 5: asm volatile("s_waitcnt vmcnt(5)" ::: "memory"); break;
+      case 6: asm volatile("s_waitcnt vmcnt(6)" ::: "memory"); break;
+      case 8: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
+      case 10: asm volatile("s_waitcnt vmcnt(10)" ::: "memory"); break;
+      case 12: asm volatile("s_waitcnt vmcnt(12)" ::: "memory"); break;
+      default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+    }
+  };
+  if constexpr (!QF) request_lead_tiles();
 
   { [[maybe_unused]] int addressed = nkblk + ntiles + wave_ntiles; SAGE_T(1, addressed); }   // tile decoded, first loads requested
   // ---- Q operand: lane (m, h) holds bytes 32*ks + 16*h .. +15 of its row for every ks ----
@@ -383,10 +422,11 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
         const int u = (lane % QUPR) ^ (r & (QUPR - 1));
         dma16(qrsrc, min(row0 + r, Lq - 1) * (int)a.q_sn * 2 + 16 * u, 0, qstage + i * 1024);
       }
+      const int behind = request_lead_tiles();   // K tiles of the lead, V scales: they may stay in flight
 #ifdef SAGE_TIMING
       const long long q_issued = __builtin_amdgcn_s_memrealtime();
 #endif
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      wait_all_but(behind);
 #ifdef SAGE_TIMING
       q_wait = __builtin_amdgcn_s_memrealtime() - q_issued;   // from the last request of the prologue to the arrival of everything
 #endif
@@ -443,11 +483,6 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
   }
 
 
-  // The other K tiles of the lead follow as soon as the raw Q rows are out of the way.
-#pragma unroll
-  for (int t = 1; t < LEAD; t++)
-    if (t < ntiles) load_k(t, dw_self);
-
   v16i bias;
 #pragma unroll
   for (int i = 0; i < 16; i++) bias[i] = kBiasBits;
@@ -487,10 +522,12 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
   // With interleaved K scales (KSUB == 3) a key's scale is picked by (n % 8) / 2 = 2*h + (r % 4) / 2: two per lane and
   // 32-key group, selected by bit 1 of the register index.
   constexpr int SUBS = KSUB == 1 ? 1 : 2;   // scale values per 32-key group and lane
-  constexpr int NSC = NT * SUBS;
+  static_assert(KW == 1 || (KSUB == 1 && (KW == 2 || KW == 4) && NT % KW == 0), "KW: 32-key groups per K scale");
+  constexpr int GPS = KW;                    // 32-key groups that share a scale
+  constexpr int NSC = NT * SUBS / GPS;
   float sc[NSC];
   auto subof = [](int r) { return KSUB == 2 ? r / 8 : KSUB == 3 ? (r >> 1) & 1 : 0; };
-  auto sci = [&](int nt, int r) { return SUBS * nt + subof(r); };
+  auto sci = [&](int nt, int r) { return (SUBS * nt + subof(r)) / GPS; };
   // K scale i of tile j as this lane needs it (before the Q scale is multiplied in)
   auto kscale_at = [&](int j, int i) -> float {
     if constexpr (KSUB == 3) {
@@ -498,10 +535,12 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
       const float lo = ksc[blk * 4 + (i & 1)], hi = ksc[blk * 4 + 2 + (i & 1)];
       return h ? hi : lo;
     } else {
-      return ksc[min((j * BN + (32 / KSUB) * i) >> a.blkk_shift, nkblk - 1)];
+      return ksc[min((j * BN + (32 / KSUB) * GPS * i) >> a.blkk_shift, nkblk - 1)];
     }
   };
   float mloc = kNegInf;
+  // Block-scaled codes: the E8M0 scale byte of this row's probabilities of the tile in flight, for the P.V phase.
+  [[maybe_unused]] int pscale = 0;
 
   // ---- S^T = K . Q^T (int8 -> int32 on the biased accumulators), then mask and row maximum ----
   auto qk = [&](int j) {
@@ -594,23 +633,36 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
     // The biased scores are positive floats (or -inf where masked), so their bit patterns order like
     // signed integers: integer max3 needs no NaN canonicalisation.
     mloc = kNegInf;
+    if constexpr (GPS > 1) {
+      // groups that share a scale share one integer chain
+#pragma unroll
+      for (int g = 0; g < NSC; g++) {
+        int mx = acc[g * GPS][0];
+#pragma unroll
+        for (int i = 1; i < 16 * GPS; i++) mx = max(mx, acc[g * GPS + i / 16][i % 16]);
+        mloc = fmaxf(mloc, __builtin_fmaf(as_f(mx), sc[g], -kBiasF * sc[g]));
+      }
+      return;
+    }
 #pragma unroll
     for (int nt = 0; nt < NT; nt++) {
 #pragma unroll
       for (int sub = 0; sub < SUBS; sub++) {
+        float smx;
         if constexpr (KSUB == 3) {
           int mx = acc[nt][2 * sub];
 #pragma unroll
           for (int r = 1; r < 16; r++)
             if (subof(r) == sub && r != 2 * sub) mx = max(mx, acc[nt][r]);
-          mloc = fmaxf(mloc, __builtin_fmaf(as_f(mx), sc[nt * SUBS + sub], -kBiasF * sc[nt * SUBS + sub]));
+          smx = __builtin_fmaf(as_f(mx), sc[nt * SUBS + sub], -kBiasF * sc[nt * SUBS + sub]);
         } else {
           constexpr int RS = 16 / KSUB;
           int mx = acc[nt][sub * RS];
 #pragma unroll
           for (int r = 1; r < RS; r++) mx = max(mx, acc[nt][sub * RS + r]);
-          mloc = fmaxf(mloc, __builtin_fmaf(as_f(mx), sc[nt * KSUB + sub], -kBiasF * sc[nt * KSUB + sub]));
+          smx = __builtin_fmaf(as_f(mx), sc[nt * KSUB + sub], -kBiasF * sc[nt * KSUB + sub]);
         }
+        mloc = fmaxf(mloc, smx);
       }
     }
   };
@@ -622,12 +674,17 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
 #pragma unroll
     for (int i = 0; i < NSC; i++) kraw[i] = kscale_at(j + 1, i);
     const float mall = xchg32_max(mloc);
-    // lazy rescale: move the reference maximum only when it grew by more than TAU
-    if (__builtin_amdgcn_ballot_w64(mall > m_used + TAU) != 0) {
+    // Block-scaled codes: the matrix pipe left the sum of the previous tile's codes in osum (unscaled: in the row-sum MFMA a
+    // scale block mixes two query rows); it joins the denominator with that tile's factor 2^(e - 8), which is the tile's
+    // E8M0 byte moved into a float's exponent field.  Then the byte may be overwritten.
+    if constexpr (FASTP) lsum = __builtin_fmaf(osum[0], as_f(pscale << 23), lsum);
+    // lazy rescale: move the reference maximum only when it grew by more than TAU (block-scaled codes: only fp32's range
+    // is at stake, and the threshold is far larger)
+    if (__builtin_amdgcn_ballot_w64(mall > m_used + (FASTP ? kBlockTau : TAU)) != 0) {
       const float m_new = fmaxf(m_used, mall);
       const float alpha = __builtin_amdgcn_exp2f(m_used - m_new);
       lsum *= alpha;
-      if constexpr (RSUM) osum[0] *= alpha;
+      if constexpr (RSUM && !FASTP) osum[0] *= alpha;
 #pragma unroll
       for (int dt = 0; dt < DTN; dt++)
 #pragma unroll
@@ -637,25 +694,35 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
     // P = exp2(S - m) * 2^PSHIFT, packed straight into the B operand of the second MFMA
     if constexpr (FASTP) {
       // The byte of an e4m3 number, read as an integer, is 8*(exponent + 7) + mantissa: piecewise linear in
-      // log2 of the value.  So y = 8*t + 56, rounded to an integer, is the fp8 code of a number within a mantissa
-      // step of 2^t, with the mantissa interpolated linearly between powers of two instead of exponentially
-      // (kCodeBias centres the error of that, at most a third of a code step).  Per score that is one v_fma_f32
-      // and three quarters of a conversion instead of v_fma_f32 + v_exp_f32 + half a v_cvt_pk_fp8_f32 (the
-      // vector ALU is the busier pipe): v_cvt_pknorm_u16_f32 turns two values x into round(65535 * x),
-      // saturating at 0 (masked scores are -inf and give code 0); with x = (256 * y + 127.5) / 65535, which the
-      // fma delivers directly, the high byte of each 16-bit result is y rounded to nearest, and one v_perm_b32
+      // log2 of the value for codes of 8 and above (the normal numbers).  So y = 8*t + 56, rounded to an integer, is
+      // the fp8 code of a number within a mantissa step of 2^t, with the mantissa interpolated linearly between powers
+      // of two instead of exponentially (kCodeBias centres the error of that, at most a third of a code step).  Per
+      // score that is one v_fma_f32 and three quarters of a conversion instead of v_fma_f32 + v_exp_f32 + half a
+      // v_cvt_pk_fp8_f32 (the vector ALU is the busier pipe): v_cvt_pknorm_u16_f32 turns two values x into
+      // round(65535 * x), saturating at 0 (masked scores are -inf and give code 0); with x = (256 * y + 127.5) / 65535,
+      // which the fma delivers directly, the high byte of each 16-bit result is y rounded to nearest, and one v_perm_b32
       // gathers the high bytes of four results into a dword of the B operand.
-      // t <= PSHIFT + TAU = 8, so the code stays <= 120 (= 256.0), below 0x7f.  The row sums of these very
-      // codes come from the matrix pipe, so numerator and denominator of O see the same values.
+      // The linear code only spans the 14.75 binades of the normal numbers (below code 8 an e4m3 byte is linear in the
+      // VALUE), so it is used block-scaled: the keys of one 128-key tile form a block per query row whose largest score
+      // lands within a binade below the top code, t = s - m - e + kBlockTop with e = ceil(row maximum of the tile - m),
+      // and the block's factor 2^e goes to the matrix pipe as the E8M0 scale of the B operand (v_mfma_scale_*: one scale
+      // byte per lane; the hardware's scale blocks are the 32-key groups, regs 0-3 / 4-7 of the two lanes of a row, and
+      // all four of a tile get the same byte here).  A key is therefore flushed to zero only when it lies 14.75 binades
+      // below the largest key of ITS tile -- not below the row's running maximum, as a statically scaled code would do,
+      // which loses a flat tail of many keys under a single large one.  The row sums of these very codes, with the
+      // same scales, come from the matrix pipe too, so numerator and denominator of O see the same values.
       constexpr float kN = 256.0f / 65535.0f, kN8 = 8.0f * kN;
       constexpr float kC = kN * (56.0f + kCodeBias) + 127.5f / 65535.0f;
-      const float k0 = __builtin_fmaf(kN8, PSHIFT - m_used, kC);
+      // (a row with no visible key in the tile has maximum -inf: the clamp gives it a finite exponent, its codes are zero)
+      const float e = fmaxf(__builtin_ceilf(mall - m_used), kBlockMinExp);
+      const float k0 = __builtin_fmaf(-kN8, e, __builtin_fmaf(kN8, kBlockTop - m_used, kC));
+      pscale = (int)(unsigned)(e + kBlockScaleBias);
 #pragma unroll
       for (int nt = 0; nt < NT; nt++) {
         float c[SUBS], mul[SUBS];
 #pragma unroll
         for (int sub = 0; sub < SUBS; sub++) {
-          mul[sub] = kN8 * sc[nt * SUBS + sub];
+          mul[sub] = kN8 * sc[(nt * SUBS + sub) / GPS];
           c[sub] = __builtin_fmaf(-kBiasF, mul[sub], k0);
         }
         float t8[16];
@@ -674,8 +741,8 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
         float c[SUBS], mul[SUBS];
 #pragma unroll
         for (int sub = 0; sub < SUBS; sub++) {
-          c[sub] = MASK ? PSHIFT - m_used : __builtin_fmaf(-kBiasF, sc[nt * SUBS + sub], PSHIFT - m_used);
-          mul[sub] = MASK ? 1.0f : sc[nt * SUBS + sub];   // masked variants already hold scores
+          c[sub] = MASK ? PSHIFT - m_used : __builtin_fmaf(-kBiasF, sc[(nt * SUBS + sub) / GPS], PSHIFT - m_used);
+          mul[sub] = MASK ? 1.0f : sc[(nt * SUBS + sub) / GPS];   // masked variants already hold scores
         }
         float p[16];
 #pragma unroll
@@ -698,8 +765,8 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
         float c[SUBS], mul[SUBS];
 #pragma unroll
         for (int sub = 0; sub < SUBS; sub++) {
-          c[sub] = MASK ? PSHIFT - m_used : __builtin_fmaf(-kBiasF, sc[nt * SUBS + sub], PSHIFT - m_used);
-          mul[sub] = MASK ? 1.0f : sc[nt * SUBS + sub];
+          c[sub] = MASK ? PSHIFT - m_used : __builtin_fmaf(-kBiasF, sc[(nt * SUBS + sub) / GPS], PSHIFT - m_used);
+          mul[sub] = MASK ? 1.0f : sc[(nt * SUBS + sub) / GPS];
         }
         // fp16 probabilities are packed in place: registers 0-7 of each accumulator take the 16 halves
         // (v_cvt_pk_f16_f32, round to nearest even) once the two scores they replace have been consumed.
@@ -741,10 +808,21 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
         v8i pb;
 #pragma unroll
         for (int e = 0; e < 8; e++) pb[e] = acc[0][8 * kk + e];
-        if constexpr (RSUM) {
-          if (dt == 0) osum = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ones, pb, osum, 0, 0, 0, 0, 0, 0);
+        if constexpr (FASTP) {
+          // block-scaled codes: byte 0 of pscale is the E8M0 scale of this row's codes, V carries 2^0.  The row sums are
+          // taken unscaled and per tile (the accumulator starts from zero at the tile's first step): the 16x16x128 form
+          // pairs lanes l and l + 16 in one column, so its 32-element scale blocks would mix two query rows.
+          if (dt == 0) {
+            const v4f zero = {0.f, 0.f, 0.f, 0.f};
+            osum = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ones, pb, kk == 0 ? zero : osum, 0, 0, 0, 0, 0, 0);
+          }
+          o[dt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vf[i], pb, o[dt], 0, 0, 0, 127, 0, pscale);
+        } else {
+          if constexpr (RSUM) {
+            if (dt == 0) osum = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ones, pb, osum, 0, 0, 0, 0, 0, 0);
+          }
+          o[dt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vf[i], pb, o[dt], 0, 0, 0, 0, 0, 0);
         }
-        o[dt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vf[i], pb, o[dt], 0, 0, 0, 0, 0, 0);
       }
       __builtin_amdgcn_sched_group_barrier(0x100, 2 * VPF, 0);
 #pragma unroll
@@ -799,22 +877,6 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
       if (j < wnt) { qk(j); rowmax(j); }
     };
     load_scales(0);
-    // Tile loads complete in the order they were requested, so waiting until only the n newest are in
-    // flight leaves exactly the requests of the last period outstanding.
-    auto wait_all_but = [&](int n) {
-      switch (n) {
-        case 0: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
-        case 1: asm volatile("s_waitcnt vmcnt(1)" ::: "memory"); break;
-        case 2: asm volatile("s_waitcnt vmcnt(2)" ::: "memory"); break;
-        case 3: asm volatile("s_waitcnt vmcnt(3)" ::: "memory"); break;
-        case 4: asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); break;
-        case 6: asm volatile("s_waitcnt vmcnt(6)" ::: "memory"); break;
-        case 8: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
-        case 10: asm volatile("s_waitcnt vmcnt(10)" ::: "memory"); break;
-        case 12: asm volatile("s_waitcnt vmcnt(12)" ::: "memory"); break;
-        default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
-      }
-    };
     auto even_barrier = [&](int j, int in_flight) {
       wait_all_but(in_flight);   // my pieces of K(j) and V(j-1) have landed
       lds_barrier();             // ... and everyone's; phase 2j-1 is over
@@ -923,7 +985,8 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
   // sum: the MFMA contracts over both key halves; it sits in lanes 0-31, lanes 32-63 hold zero and get it from
   // their partner); the fp32 sum of the unrounded ones serves LSE only.
   float msum = 0.f;
-  if constexpr (RSUM) msum = xchg32_sum(osum[0]);
+  if constexpr (FASTP) msum = xchg32_sum(__builtin_fmaf(osum[0], as_f(pscale << 23), lsum));   // the last tile's sum is still pending
+  else if constexpr (RSUM) msum = xchg32_sum(osum[0]);
   if constexpr (MSUM) lsum = msum;
   else lsum = xchg32_sum(lsum);
   const float den = RSUM ? msum : lsum;
@@ -1010,10 +1073,10 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
 }
 
 
-template <int D, int NW, int BN, int PV, bool CAUSAL, bool MSUM, int MASK, int KSUB = 1, bool QF = false>
+template <int D, int NW, int BN, int PV, bool CAUSAL, bool MSUM, int MASK, int KSUB = 1, bool QF = false, int KW = 1>
 static hipError_t launch_one(const AttnArgs& a, int grid, hipStream_t st) {
   constexpr int smem = attn_lds_bytes<D, NW, BN, PV, CAUSAL, QF>();
-  auto kern = attn_kernel<D, NW, BN, PV, CAUSAL, MSUM, MASK, KSUB, QF>;
+  auto kern = attn_kernel<D, NW, BN, PV, CAUSAL, MSUM, MASK, KSUB, QF, KW>;
   // More than 64 KB of dynamic LDS has to be allowed once per kernel and device.
   constexpr int kMaxDevices = 64;
   static std::atomic<bool> attr_done[kMaxDevices] = {};   // (two host threads may make the first call at once: setting it twice is harmless)

@@ -8,9 +8,11 @@ namespace sage {
 
 hipError_t launch_attn_qfused(const AttnArgs& a, int D, int pv, bool causal, int grid, hipStream_t st) {
   const bool msum = a.lse == nullptr;
-#define SAGE_ATTN_Q(DD, PVV, BNN, MS) (causal ? launch_one<DD, 8, BNN, PVV, true, MS, 0, 1, true>(a, grid, st) : launch_one<DD, 8, BNN, PVV, false, MS, 0, 1, true>(a, grid, st))
+#define SAGE_ATTN_QW(DD, PVV, BNN, MS, KWW) (causal ? launch_one<DD, 8, BNN, PVV, true, MS, 0, 1, true, KWW>(a, grid, st) : launch_one<DD, 8, BNN, PVV, false, MS, 0, 1, true, KWW>(a, grid, st))
+#define SAGE_ATTN_Q(DD, PVV, BNN, MS) (a.blkk >= 128 ? SAGE_ATTN_QW(DD, PVV, BNN, MS, 4) : a.blkk == 64 ? SAGE_ATTN_QW(DD, PVV, BNN, MS, 2) : SAGE_ATTN_QW(DD, PVV, BNN, MS, 1))
   if (D == 128) return pv ? (msum ? SAGE_ATTN_Q(128, 1, 128, true) : SAGE_ATTN_Q(128, 1, 128, false)) : SAGE_ATTN_Q(128, 0, 128, false);
   return pv ? (msum ? SAGE_ATTN_Q(64, 1, 128, true) : SAGE_ATTN_Q(64, 1, 128, false)) : (msum ? SAGE_ATTN_Q(64, 0, 128, true) : SAGE_ATTN_Q(64, 0, 128, false));
+#undef SAGE_ATTN_QW
 #undef SAGE_ATTN_Q
 }
 

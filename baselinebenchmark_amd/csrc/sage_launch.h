@@ -46,6 +46,27 @@ struct PrepVArgs {
   int64_t panel_sh;
 };
 
+// Division of a 32-bit unsigned number by a launch constant as a multiply-high and two shifts (exact for every 32-bit
+// dividend): the tile decode of the attention kernel divides the workgroup index by head counts that are no powers of
+// two, and a true integer division is some twenty dependent instructions on this hardware, paid by every workgroup
+// before its first memory request.
+struct FastDiv {
+  uint32_t mul, sh1, sh2;
+};
+inline FastDiv make_fastdiv(uint32_t d) {
+  FastDiv f;
+  uint32_t L = 0;
+  while (L < 32 && (uint64_t(1) << L) < d) L++;               // ceil(log2 d); d >= 1
+  f.mul = (uint32_t)(((uint64_t(1) << 32) * ((uint64_t(1) << L) - d)) / d + 1);
+  f.sh1 = L < 1 ? L : 1;
+  f.sh2 = L < 1 ? 0 : L - 1;
+  return f;
+}
+__device__ inline uint32_t fastdiv(uint32_t n, const FastDiv& f) {
+  const uint32_t t = __umulhi(f.mul, n);
+  return (t + ((n - t) >> f.sh1)) >> f.sh2;
+}
+
 struct AttnArgs {
   const int8_t* q;
   const int8_t* k;
@@ -63,6 +84,11 @@ struct AttnArgs {
   int k_interleave;          // 1: four interleaved K scales per block (scale t for the keys n with (n % 8) / 2 == t); host-side dispatch only
   int out_bf16;
   int nqt;  // q-tiles per sequence (fixed-length mode)
+  // launch constants of the tile decode (filled in by finish_attn_args)
+  int G;                    // q-heads per KV head
+  int tier_shift;           // fixed-length mode, per-XCD tile order: log2 of the widest range of q-tiles; -1: plain order
+  FastDiv div_G, div_Hkv, div_heads;   // heads = B*Hq (fixed-length) or Hq (packed)
+  FastDiv div_range, div_last;         // full-attention tile order: q-tiles x heads-per-XCD of a range; width of the last range
   // packed mode (cu_q != nullptr)
   const int32_t* cu_q;
   const int32_t* cu_k;
@@ -99,6 +125,8 @@ hipError_t launch_prepass_small(const QuantArgs& qa, const PrepVArgs& va, int dt
                                 void* km_out, float* vscale_out, hipStream_t st);
 
 AttnConfig attn_config(int D, int pv, bool packed);
+// Fills in the launch constants of the tile decode from the dimensions already in `a` (B, Hq, Hkv, nqt, cu_q).
+void finish_attn_args(AttnArgs& a, bool causal);
 hipError_t launch_attn(const AttnArgs& a, int D, int pv, bool causal, int grid, hipStream_t st);
 hipError_t launch_attn_masked(const AttnArgs& a, int D, int pv, int grid, hipStream_t st);
 hipError_t launch_attn_qfused(const AttnArgs& a, int D, int pv, bool causal, int grid, hipStream_t st);

@@ -12,8 +12,11 @@ output type instead:
     some row of its group grew by more than tau = 3 over it (lazy rescale), then o and the row sum are scaled by
     exp2(old - new);
   * P = 2^5 * exp2(s - m) rounded to e4m3 (round to nearest even) -- or, for the kernels that need no LSE and no
-    explicit mask, the "linear-mantissa" code: 8 * t + 56 - 0.3, t = s - m + 5, rounded to nearest (as the high byte of a
-    16-bit conversion of (256 * code + 127.5) / 65535) and read as an e4m3 byte;
+    explicit mask, the block-scaled "linear-mantissa" code: the keys of a 128-key tile form one block per query row with
+    the exponent e = max(ceil(row maximum of the tile - m), -110); the code is 8 * t + 56 - 0.3, t = s - m - e + 8.75,
+    rounded to nearest (as the high byte of a 16-bit conversion of (256 * code + 127.5) / 65535) and read as an e4m3
+    byte, and the matrix pipe multiplies the block by 2^(e - 8) (its E8M0 scale operand).  There the reference maximum
+    moves when a row's tile maximum exceeds it by more than 20;
   * O = sum P8 * V8 and the denominator sum P8 (of the very same rounded values), fp32 accumulation on the GPU,
     float64 here; out = O / den * v_scale;  LSE2 = m + log2(sum of the unrounded p) - 5.
 
@@ -31,6 +34,10 @@ BIAS = np.float32(12582912.0)      # 1.5 * 2^23: the INT32 accumulators start fr
 PSHIFT = np.float32(5.0)
 TAU = np.float32(3.0)
 CODE_BIAS = np.float32(-0.3)
+BLOCK_TOP = np.float32(8.75)       # the block maximum is coded within one binade below 2^8.75 (code <= 126 = 448)
+BLOCK_TAU = np.float32(20.0)
+BLOCK_MIN_EXP = np.float32(-110.0)
+BLOCK_SCALE_BIAS = 119             # E8M0 byte of a block = 119 + e: the matrix pipe applies 2^(e - 8)
 M_INIT = np.float32(-1.0e30)
 KN = np.float32(256.0) / np.float32(65535.0)                      # code units -> units of the 16-bit conversion
 KN8 = np.float32(8.0) * KN
@@ -51,18 +58,27 @@ def decode_e4m3(code: np.ndarray) -> np.ndarray:
     return np.where(e == 0, m * 2.0 ** -9, np.exp2((e - 7).astype(np.float64)) * (1.0 + m / 8.0))
 
 
-def linear_code_of(acc: np.ndarray, sc: np.ndarray, base: np.ndarray) -> np.ndarray:
-    """The kernel's linear-mantissa code of 2^t, t = (acc - BIAS) * sc + base: y = 8 * t + 56 + CODE_BIAS rounded to
-    nearest, computed the kernel's way (baselinebenchmark_amd/csrc/sage_attn_kernel.h, softmax): fp32 FMAs deliver
-    x = (256 * y + 127.5) / 65535, the 16-bit conversion gives rne(65535 * x) saturated to [0, 65535], and the code is
-    its high byte.  acc [R, N] biased fp32 accumulators, sc [R, N] fp32 scale products, base [R] fp32."""
-    k0 = _fma32(KN8, base, KC)
+def linear_code_of(acc: np.ndarray, sc: np.ndarray, k0b: np.ndarray) -> np.ndarray:
+    """The kernel's linear-mantissa code of 2^t: y = 8 * t + 56 + CODE_BIAS rounded to nearest, computed the kernel's way
+    (baselinebenchmark_amd/csrc/sage_attn_kernel.h, softmax): fp32 FMAs deliver x = (256 * y + 127.5) / 65535, the 16-bit
+    conversion gives rne(65535 * x) saturated to [0, 65535], and the code is its high byte.  acc [R, N] biased fp32
+    accumulators, sc [R, N] fp32 scale products, k0b [R] the per-row constant of the tile (block_constants)."""
     mul = (KN8 * sc).astype(np.float32)
-    c = _fma32(-BIAS, mul, k0[:, None])
-    x = _fma32(acc, mul, c)
+    c = _fma32(-BIAS, mul, k0b[:, None])
     with np.errstate(invalid="ignore"):
+        x = _fma32(acc, mul, c)
         u16 = np.rint(np.clip(x.astype(np.float64), 0.0, 1.0) * 65535.0)
-    return np.floor(u16 / 256.0)
+    return np.where(np.isnan(u16), 0.0, np.floor(u16 / 256.0))
+
+
+def block_constants(bmax: np.ndarray, m_used: np.ndarray):
+    """Per row: the block exponent e = max(ceil(bmax - m), -110) and the fma constant of the code, both in fp32 as the
+    kernel computes them.  bmax [R] fp32 maxima of the row's scores in the tile (-inf without visible keys), m_used [R]."""
+    with np.errstate(invalid="ignore"):
+        d = (bmax - m_used).astype(np.float32)
+        e = np.maximum(np.ceil(d), BLOCK_MIN_EXP).astype(np.float32)
+    k0 = _fma32(KN8, (BLOCK_TOP - m_used).astype(np.float32), KC)
+    return e, _fma32(-KN8, e, k0)
 
 
 def _rne_e4m3(p32: np.ndarray) -> np.ndarray:
@@ -72,8 +88,11 @@ def _rne_e4m3(p32: np.ndarray) -> np.ndarray:
 
 
 def fp8_attention_model(q_int8, k_int8, v, q_scale, k_scale, tensor_layout="HND", BLKQ=128, BLKK=64, is_causal=False,
-                        attn_mask=None, mask_mult=1.0, linear_code=None, want_lse=False):
+                        attn_mask=None, mask_mult=1.0, linear_code=None, want_lse=False, row_offset=0):
     """Returns (out float64 [layout of q], lse2 float64 [B,Hq,Sq] or None).
+
+    ``row_offset``: q_int8 / q_scale hold the query rows row_offset, row_offset + 1, ... of a longer problem (a multiple
+    of 32 and of BLKQ, so that wavefront groups and scale blocks keep their places); it only moves the causal diagonal.
 
     ``linear_code``: None picks what the library picks (the linear-mantissa code when neither a mask nor LSE is
     asked for, exact exp2 + e4m3 rounding otherwise).  ``attn_mask``: bool (True keeps) or additive, already
@@ -99,6 +118,8 @@ def fp8_attention_model(q_int8, k_int8, v, q_scale, k_scale, tensor_layout="HND"
     out = np.zeros((B, Hq, Sq, D), np.float64)
     lse = np.full((B, Hq, Sq), -np.inf, np.float64)
     rows = np.arange(Sq)
+    assert row_offset % GROUP == 0 and row_offset % BLKQ == 0
+    rows_abs = rows + row_offset
     ngroups = (Sq + GROUP - 1) // GROUP
     gidx = rows // GROUP
     for b in range(B):
@@ -110,13 +131,15 @@ def fp8_attention_model(q_int8, k_int8, v, q_scale, k_scale, tensor_layout="HND"
             den = np.zeros(Sq, np.float64)
             lsum = np.zeros(Sq, np.float64)
             for n0 in range(0, Skv, TILE):
+                if is_causal and n0 > rows_abs[-1]:
+                    break                                    # tiles above the diagonal: skipped, as in the kernel
                 n1 = min(n0 + TILE, Skv)
                 keys = np.arange(n0, n1)
                 sc = (qrow_scale[:, None] * ks[b, hk][keys // BLKK][None, :]).astype(np.float32)   # fp32 product
                 acc = (BIAS.astype(np.float64) + qi[b, hq] @ ki[b, hk, n0:n1].T).astype(np.float32)   # exact: |dot| < 2^22
                 dead = np.zeros((Sq, n1 - n0), bool)
                 if is_causal:
-                    dead |= keys[None, :] > rows[:, None]
+                    dead |= keys[None, :] > rows_abs[:, None]
                 if masked:
                     sv = _fma32(acc, sc, (-BIAS * sc).astype(np.float32))
                     mk = mask[b, hq][:, n0:n1]
@@ -131,7 +154,7 @@ def fp8_attention_model(q_int8, k_int8, v, q_scale, k_scale, tensor_layout="HND"
                     score = _fma32(acc, sc, (-BIAS * sc).astype(np.float32))
                     mloc = np.where(dead, -np.inf, score).max(axis=1).astype(np.float32)
                 # lazy rescale, decided per group of 32 rows
-                grew = mloc > (m_used + TAU).astype(np.float32)
+                grew = mloc > (m_used + (BLOCK_TAU if linear_code else TAU)).astype(np.float32)
                 trig = np.zeros(ngroups, bool)
                 np.logical_or.at(trig, gidx, grew)
                 upd = trig[gidx]
@@ -143,9 +166,10 @@ def fp8_attention_model(q_int8, k_int8, v, q_scale, k_scale, tensor_layout="HND"
                 m_used = m_new
                 base = (PSHIFT - m_used).astype(np.float32)                       # [Sq]
                 if linear_code:
-                    code = linear_code_of(acc, sc, base)
+                    e, k0b = block_constants(mloc, m_used)
+                    code = linear_code_of(acc, sc, k0b)
                     code = np.where(dead, 0, code)
-                    p8 = decode_e4m3(code)
+                    p8 = decode_e4m3(code) * np.exp2(e.astype(np.float64) - 8.0)[:, None]
                 else:
                     if masked:
                         with np.errstate(invalid="ignore"):

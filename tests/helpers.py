@@ -57,3 +57,27 @@ def sageattn_cabi(q, k, v, out, *, layout="HND", is_causal=False, pv="fp16", BLK
     nbytes = lib.sage_sageattn_workspace_bytes(B, Hq, Hkv, Sq, Skv, D, BLKQ, BLKK, pvm, 0, 0, 0)
     ws = workspace if workspace is not None else torch.empty(max(nbytes, 256), device=q.device, dtype=torch.uint8)
     return lib.sage_sageattn(P(q), P(k), P(v), P(out), P(lse), P(ws), ws.numel(), *tail)
+
+
+def check_rows_fp8(got, q_rows, k1, v1, r0, blkq, blkk, causal, out_dtype):
+    """Rows r0 .. r0 + T of ONE (batch, head) of a long FP8 P.V problem against the oracle, host cost O(T * S):
+    got [T, D] (the library's output rows), q_rows [T, D], k1 / v1 [S, D] raw operands of that head (K smoothed with its
+    own mean, per-block INT8 by the oracle's quantiser, V per-channel e4m3).  Returns the metrics against
+    (a) the exact-softmax formula on the same quantised operands, (b) the kernel's arithmetic model, (c) FP32 SDPA on
+    the raw operands."""
+    from oracle import attention as oa
+    from oracle import fp8_model as fm
+    from oracle import quant as oq
+    T, S = q_rows.shape[0], k1.shape[0]
+    q4, k4, v4 = q_rows[None, None].cpu(), k1[None, None].cpu(), v1[None, None].cpu()
+    qi, qs, ki, ks = oq.per_block_int8(q4, k4, km=oq.k_mean(k4), BLKQ=blkq, BLKK=blkk)
+    v8, vsc = oq.quant_v_fp8(v4)
+    vis = (torch.arange(S)[None, :] <= torch.arange(r0, r0 + T)[:, None])[None, None] if causal else None
+    ref, _ = oa.sage_reference(qi, ki, v8, qs, ks, "HND", blkq, blkk, attn_mask=vis, v_scale=vsc)
+    model, _ = fm.fp8_attention_model(qi, ki, v4, qs, ks, "HND", blkq, blkk, is_causal=causal, row_offset=r0)
+    logits = (q4.double() @ k4.double().transpose(-1, -2)) * (q4.shape[-1] ** -0.5)
+    if causal:
+        logits = logits.masked_fill(~vis, -float("inf"))
+    sdpa = torch.softmax(logits, dim=-1) @ v4.double()
+    g = got.detach().cpu().float()[None, None]
+    return oa.metrics(g, ref), oa.metrics(g, model), oa.metrics(g, sdpa.float())

@@ -19,7 +19,7 @@ import torch
 import baselinebenchmark_amd as sa
 from oracle import attention as oa
 from oracle import quant as oq
-from tests.helpers import randn, shape4
+from tests.helpers import check_rows_fp8, randn, shape4
 
 pytestmark = [pytest.mark.gpu, pytest.mark.sage_attention]
 DEV = "cuda"
@@ -207,7 +207,19 @@ def test_long_sequence_properties_full_size_head():
     out3, _ = sa.forward(qi, ki, vg, qs, ks, output_dtype=torch.bfloat16, BLKQ=64, BLKK=128, is_causal=True, pv_mode="fp8")
     out4, _ = sa.forward(qi, ki, vg * 2, qs, ks, output_dtype=torch.bfloat16, BLKQ=64, BLKK=128, is_causal=True, pv_mode="fp8")
     assert torch.equal(out4.cpu().float(), out3.cpu().float() * 2)
-    assert oa.metrics(out3.cpu().float(), o)["cosine"] >= 0.999
+    o3 = out3.cpu().float()
+    # (two kernels whose probabilities are rounded to three mantissa bits in different ways -- exact e4m3 rounding
+    # against the linear-mantissa code -- each about 0.9997 from the formula: between themselves 0.9993-0.9994.  The bar
+    # for either one is the oracle, below.)
+    assert oa.metrics(o3, o)["cosine"] >= 0.999
+    # ... and that kernel (linear-mantissa, block-scaled codes: the one the benchmark times) against the oracle at this
+    # length: the prefix and the last rows against the exact-softmax formula, the last rows against the arithmetic model
+    assert oa.metrics(o3[:, :, :P], ref)["cosine"] >= 0.999
+    assert oa.metrics(o3[:, :, S - T:], ref_t)["cosine"] >= 0.999
+    for hq in range(2):
+        m_ref, m_model, m_sdpa = check_rows_fp8(out3[0, hq, S - T:], q[0, hq, S - T:], k[0, 0], v[0, 0], S - T, 64, 128, True,
+                                                torch.bfloat16)
+        assert m_ref["cosine"] >= 0.999 and m_model["rel_rmse"] < 2.5e-3 and m_sdpa["cosine"] >= 0.999, (m_ref, m_model, m_sdpa)
 
 
 def test_lse_is_empty_unless_requested():
@@ -551,6 +563,15 @@ def test_config2_full_size_properties():
     lim = (cut // 256) * 256
     assert torch.equal(pert[:, :, :lim], base[:, :, :lim])
     assert not torch.equal(pert[:, :, lim + 256:], base[:, :, lim + 256:])
+    del base, pert, k2, v2
+    # the benchmarked call itself against the oracle, on row slices of two (batch, head) pairs (host cost 256 x 16384 each)
+    S = q.shape[2]
+    for b, h, r0 in ((0, 0, S - 256), (1, 31, 8192), (1, 5, 256)):
+        m_ref, m_model, m_sdpa = check_rows_fp8(out[b, h, r0:r0 + 256], q[b, h, r0:r0 + 256], k[b, h], v[b, h], r0, 64, 128, True,
+                                                torch.bfloat16)
+        print(f"c2 rows {r0}..{r0 + 256} of ({b},{h}): cos vs formula {m_ref['cosine']:.6f}, rel-RMSE vs model {m_model['rel_rmse']:.2e}, "
+              f"cos vs FP32 SDPA {m_sdpa['cosine']:.6f} max-abs {m_sdpa['max_abs']:.4f}")
+        assert m_ref["cosine"] >= 0.999 and m_model["rel_rmse"] < 2.5e-3 and m_sdpa["cosine"] >= 0.999, (b, h, r0, m_ref, m_model, m_sdpa)
 
 
 def test_config3_full_size_properties():
@@ -572,6 +593,18 @@ def test_config3_full_size_properties():
     start = (S // 256) * 256
     tail = sa.sageattn(w.q[:, start:].contiguous(), w.k, w.v, **w.kwargs)
     assert torch.equal(tail, out[:, start:])
+    del tail
+    # the last (partial) q-tile and a middle one of two heads against the oracle (host cost 256 x 32760 each).  The x20
+    # outlier channels in q AND k make per-block INT8 itself coarse (the formula on the quantised operands is what the
+    # kernel must match); the distance to FP32 SDPA on the raw operands is reported and held to the looser bound it meets.
+    pairs = w.q[0, :8].float().abs().amax(dim=0)              # [H, D]: heads with an outlier channel show up here
+    hot = int((pairs.amax(dim=1) > 40).nonzero()[0]) if (pairs.amax(dim=1) > 40).any() else 0
+    for h, r0, T in ((hot, start, S - start), (23 if hot != 23 else 0, 16384, 256)):
+        m_ref, m_model, m_sdpa = check_rows_fp8(out[0, r0:r0 + T, h], w.q[0, r0:r0 + T, h], w.k[0, :, h], w.v[0, :, h], r0, 128, 64,
+                                                False, torch.bfloat16)
+        print(f"c3 rows {r0}..{r0 + T} of head {h}: cos vs formula {m_ref['cosine']:.6f}, rel-RMSE vs model {m_model['rel_rmse']:.2e}, "
+              f"cos vs FP32 SDPA {m_sdpa['cosine']:.6f} max-abs {m_sdpa['max_abs']:.4f}")
+        assert m_ref["cosine"] >= 0.999 and m_model["rel_rmse"] < 2.5e-3 and m_sdpa["cosine"] >= 0.99, (h, r0, m_ref, m_model, m_sdpa)
 
 
 def test_sageattn_with_the_external_quant_recipe():

@@ -2,7 +2,8 @@
 
 The other FP8 tests compare with the exact-softmax formula on unquantised V at cosine >= 0.999 -- a bound on the
 ALGORITHM (e4m3 P and V).  Here the kernel's own arithmetic is checked: same quantised V, same reference-maximum
-walk (tiles of 128 keys, groups of 32 rows, tau = 3), same fp8 code for P, denominator from the rounded values.  What
+walk (tiles of 128 keys, groups of 32 rows, lazy rescale), same fp8 code for P (block-scaled where the library uses
+the linear-mantissa code), denominator from the rounded values.  What
 is left between kernel and model is the fp32 accumulation order and the rounding of the output type, so the bound is
 the output type's: relative RMSE < 6e-4 for fp16 outputs (half an ulp is 2.4e-4 worst case, 1.4e-4 rms) and < 2.5e-3
 for bf16 outputs (1.1e-3 rms), |LSE2 error| < 2e-4.
@@ -92,6 +93,32 @@ def test_single_query_row_with_an_additive_mask():
         v8, vsc = oq.quant_v_fp8(vc)
         want = (v8.double() * vsc.double()[:, :, None, :])[:, :, :1].expand(1, 2, 1, 128)
         assert torch.allclose(outc.cpu().double(), want, rtol=2 ** -10, atol=1e-6), trial
+
+
+@pytest.mark.parametrize("binades", [9.5, 11.5, 12.5, 13.5, 15.5, 30.0])
+@pytest.mark.parametrize("lse", [False, True], ids=["linear-code", "exact-exp2-lse"])
+def test_one_large_key_above_a_flat_tail(binades, lse):
+    """An attention sink over a flat tail: key 0 lies `binades` above 8191 equal keys, which together carry most of the
+    softmax mass.  Gated on the relative RMSE against the exact-softmax formula (a cosine hardly notices a lost tail).  The
+    block-scaled linear code keeps three mantissa bits at any distance; the exact-exponential kernels (LSE wanted) code P
+    against the row maximum and lose the tail where e4m3's 18 binades end, which is stated here as their bound."""
+    S, D, Sq = 8192, 64, 32
+    qi = torch.zeros(1, 1, Sq, D, dtype=torch.int8)
+    qi[..., 0] = 100
+    ki = torch.zeros(1, 1, S, D, dtype=torch.int8)
+    ki[0, 0, 0, 0] = 100
+    qs, ks = torch.full((1, 1, 1), binades / 10000.0), torch.ones(1, 1, S // 64)
+    v = torch.randn(1, 1, S, D, generator=torch.Generator().manual_seed(3)).to(torch.float16)
+    out, _ = sa.forward(qi.to(DEV), ki.to(DEV), v.to(DEV), qs.to(DEV), ks.to(DEV), return_lse=lse, pv_mode="fp8")
+    v8, vsc = oq.quant_v_fp8(v)
+    ref, _ = oa.sage_reference(qi, ki, v8, qs, ks, "HND", 128, 64, v_scale=vsc)
+    model, _ = fm.fp8_attention_model(qi, ki, v, qs, ks, "HND", 128, 64, want_lse=lse)
+    _check(out, model, torch.float16, (binades, lse))
+    err = oa.metrics(out.cpu().float(), ref)["rel_rmse"]
+    if not lse:
+        assert err < 0.02, err
+    else:
+        assert err < (0.06 if binades <= 12.5 else 0.2 if binades <= 15.5 else 1.01), err
 
 
 def test_one_call_pipeline_fp8_matches_the_model():

@@ -54,7 +54,8 @@ def test_linear_code_by_way_of_the_16_bit_conversion_is_the_code_value_rounded_t
     acc = (12582912.0 + dots).astype(np.float32)
     sc = np.broadcast_to(rng.uniform(1e-4, 3e-4, size=(R, 1)).astype(np.float32), (R, N))
     base = (5.0 - (dots.max(axis=1) * sc[:, 0].astype(np.float64))).astype(np.float32) + rng.uniform(0, 3, R).astype(np.float32)
-    code = fm.linear_code_of(acc, sc, base)
+    k0 = fm._fma32(fm.KN8, base, fm.KC)                       # the constant of a block with exponent 0
+    code = fm.linear_code_of(acc, sc, k0)
     y = 8.0 * (dots * sc.astype(np.float64) + base[:, None].astype(np.float64)) + 56.0 - 0.3
     want = np.clip(np.rint(y), 0, 255)
     near_tie = np.abs(y - np.floor(y) - 0.5) < 0.02
@@ -63,14 +64,23 @@ def test_linear_code_by_way_of_the_16_bit_conversion_is_the_code_value_rounded_t
     assert (np.abs(code - want) <= 1).all()
 
 
+def _e4m3_value(code):
+    return float(torch.tensor([code], dtype=torch.uint8).view(torch.float8_e4m3fn).float())
+
+
 @pytest.mark.parametrize("linear", [False, True])
 def test_one_tile_closed_form_with_scalar_loops(linear):
     """Skv <= 128: one tile, the reference maximum is the row's own maximum, so the model must equal
-    sum_j P8_j V8_j / sum_j P8_j * v_scale with P8 computed score by score from the INT32 dot products."""
+    sum_j P8_j V8_j / sum_j P8_j * v_scale with P8 computed score by score from the INT32 dot products.  Block-scaled
+    codes: the tile is one block per row with the exponent e = max(ceil(row maximum - m), -110) (0 here, the reference
+    maximum being the row maximum), the code that of 2^(s - m - e + 8.75), its weight 2^(e - 8)."""
     q, k, v, qi, qs, ki, ks = _quantised("HND", 1, 2, 1, 5, 9, 64, 11)
     out, lse = fm.fp8_attention_model(qi, ki, v, qs, ks, "HND", 64, 128, linear_code=linear, want_lse=not linear)
     v8, vsc = oq.quant_v_fp8(v)
     v8 = v8.float()
+    kn = _f32(256.0 / 65535.0)
+    kn8 = _f32(8.0 * kn)
+    kc = _f32(_f32(kn * _f32(56.0 - 0.3)) + _f32(127.5 / 65535.0))
     for h in range(2):
         for i in range(5):
             sc = _f32(float(qs[0, h, 0]) * float(ks[0, 0, 0]))
@@ -80,13 +90,17 @@ def test_one_tile_closed_form_with_scalar_loops(linear):
             m = max(scores)
             base = _f32(5.0 - m)
             p8, praw = [], []
-            for d in dots:
+            for j, d in enumerate(dots):
                 if linear:
-                    k0 = _f32(_f32(8.0 * base) + _f32(56.0 - 0.3))
-                    c = _f32(-12582912.0 * (8.0 * sc) + k0)
-                    t8 = _f32((12582912.0 + d) * (8.0 * sc) + c)
-                    code = min(max(int(np.rint(t8)), 0), 255)
-                    p8.append(float(torch.tensor([code], dtype=torch.uint8).view(torch.float8_e4m3fn).float()))
+                    e = max(math.ceil(_f32(max(scores) - m)), -110)
+                    k0 = _f32(kn8 * _f32(8.75 - m) + kc)
+                    k0b = _f32(-kn8 * e + k0)
+                    mul = _f32(kn8 * sc)
+                    c = _f32(-12582912.0 * mul + k0b)
+                    x = _f32((12582912.0 + d) * mul + c)
+                    code = int(np.rint(min(max(x, 0.0), 1.0) * 65535.0)) >> 8
+                    assert code <= 126
+                    p8.append(_e4m3_value(code) * 2.0 ** (e - 8))
                 else:
                     c = _f32(-12582912.0 * sc + base)
                     p = _f32(2.0 ** _f32((12582912.0 + d) * sc + c))
@@ -98,6 +112,53 @@ def test_one_tile_closed_form_with_scalar_loops(linear):
                 assert abs(out[0, h, i, ch].item() - val) < 1e-12 * max(1.0, abs(val)) + 1e-12
             if not linear:
                 assert abs(lse[0, h, i].item() - (m + math.log2(sum(praw)) - 5.0)) < 1e-9
+
+
+def test_block_scaled_codes_use_the_top_of_the_range_in_every_tile():
+    """The largest score of a row in a tile is coded within one binade below 2^8.75: codes 118 ... 126, never the NaN
+    byte, however far the tile lies below (or, within the lazy-rescale margin, above) the reference maximum."""
+    rng = np.random.default_rng(6)
+    R, N = 64, 128
+    dots = rng.integers(-40000, 40000, size=(R, N))
+    acc = (12582912.0 + dots).astype(np.float32)
+    sc = np.broadcast_to(rng.uniform(1e-4, 3e-4, size=(R, 1)).astype(np.float32), (R, N))
+    score = fm._fma32(acc, sc, (-fm.BIAS * sc).astype(np.float32))
+    bmax = score.max(axis=1)
+    for lag in (-20.0, -3.0, 0.0, 17.5, 60.0, 200.0):                     # reference maximum minus the tile's maximum
+        m_used = (bmax + np.float32(lag) + rng.uniform(0, 1, R).astype(np.float32)).astype(np.float32)
+        e, k0b = fm.block_constants(bmax, m_used)
+        code = fm.linear_code_of(acc, sc, k0b)
+        top = code.max(axis=1)
+        if lag <= 100:
+            assert (e == np.ceil(bmax - m_used)).all()
+            assert (top >= 118).all() and (top <= 126).all(), lag
+            # the value a code stands for, with its block's factor, is 2^(s - m + 0.75) within a mantissa step
+            val = fm.decode_e4m3(code) * np.exp2(e.astype(np.float64) - 8.0)[:, None]
+            want = np.exp2(score.astype(np.float64) - m_used[:, None] + 0.75)
+            live = code >= 8
+            assert live.mean() > 0.3 and (np.abs(val[live] / want[live] - 1) < 0.13).all()
+        else:
+            assert (e == -110).all() and (code == 0).all()              # 2^-200 of the maximum: flushed, exponent clamped
+
+
+@pytest.mark.parametrize("binades", [9.5, 11.5, 12.5, 13.5, 15.5, 30.0])
+def test_one_large_key_above_a_flat_tail(binades):
+    """A single key `binades` above 8191 equal ones (an attention sink over a flat tail): the tail carries most of the
+    softmax mass although each of its keys is tiny next to the row maximum.  A code scaled to the row maximum alone
+    flushes or mis-codes the tail from about 12 binades on (e4m3 has 18); block-scaled codes keep every tile at the top
+    of the range, so only the 127 tail keys that share the large key's tile are lost and the error stays that of three
+    mantissa bits at any distance."""
+    S, D, Sq = 8192, 64, 32
+    qi = torch.zeros(1, 1, Sq, D, dtype=torch.int8)
+    qi[..., 0] = 100
+    ki = torch.zeros(1, 1, S, D, dtype=torch.int8)
+    ki[0, 0, 0, 0] = 100
+    qs, ks = torch.full((1, 1, 1), binades / 10000.0), torch.ones(1, 1, S // 64)
+    v = torch.randn(1, 1, S, D, generator=torch.Generator().manual_seed(3)).to(torch.bfloat16)
+    v8, vsc = oq.quant_v_fp8(v)
+    ref, _ = oa.sage_reference(qi, ki, v8, qs, ks, "HND", 128, 64, v_scale=vsc)
+    lin, _ = fm.fp8_attention_model(qi, ki, v, qs, ks, "HND", 128, 64, linear_code=True)
+    assert oa.metrics(lin, ref)["rel_rmse"] < 0.02
 
 
 @pytest.mark.parametrize("linear", [False, True])
