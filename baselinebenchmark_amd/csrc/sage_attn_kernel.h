@@ -637,9 +637,17 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
       // groups that share a scale share one integer chain
 #pragma unroll
       for (int g = 0; g < NSC; g++) {
-        int mx = acc[g * GPS][0];
+        // (one chain per 32-key group, combined at the end: independent chains issue back to back)
+        int mxg[GPS];
 #pragma unroll
-        for (int i = 1; i < 16 * GPS; i++) mx = max(mx, acc[g * GPS + i / 16][i % 16]);
+        for (int t = 0; t < GPS; t++) {
+          mxg[t] = acc[g * GPS + t][0];
+#pragma unroll
+          for (int r = 1; r < 16; r++) mxg[t] = max(mxg[t], acc[g * GPS + t][r]);
+        }
+        int mx = mxg[0];
+#pragma unroll
+        for (int t = 1; t < GPS; t++) mx = max(mx, mxg[t]);
         mloc = fmaxf(mloc, __builtin_fmaf(as_f(mx), sc[g], -kBiasF * sc[g]));
       }
       return;
