@@ -83,9 +83,9 @@ __device__ __forceinline__ void quant_int8_tile(const QuantArgs& a, const int bl
     raw[p][0] = raw[p][1] = make_uint4(0, 0, 0, 0);
     float dsum = 0.f;
     if (r < rows) {
-      const uint4* src = reinterpret_cast<const uint4*>(a.x + xbase + (int64_t)(n0 + r) * a.x_sn + tc * 16);
-      raw[p][0] = src[0];
-      raw[p][1] = src[1];
+      const u16* src = a.x + xbase + (int64_t)(n0 + r) * a.x_sn + tc * 16;
+      raw[p][0] = load_stream16(src);
+      raw[p][1] = load_stream16(src + 8);
       if (has_km) {
         const u16* e = reinterpret_cast<const u16*>(raw[p]);
         uint32_t d[8];
@@ -161,7 +161,7 @@ __device__ __forceinline__ void quant_int8_tile(const QuantArgs& a, const int bl
         int q = (int)z;  // truncation toward zero
         packed[i >> 2] |= (uint32_t)(q & 0xff) << (8 * (i & 3));
       }
-      *reinterpret_cast<uint4*>(a.out + obase + (int64_t)(n0 + r) * a.o_sn + tc * 16) = make_uint4(packed[0], packed[1], packed[2], packed[3]);
+      store_stream16(a.out + obase + (int64_t)(n0 + r) * a.o_sn + tc * 16, make_uint4(packed[0], packed[1], packed[2], packed[3]));
     }
   }
 }
@@ -200,8 +200,7 @@ __global__ void __launch_bounds__(256) colstat_partial_kernel(ColStatArgs a) {
   acc_t acc[8];
 #pragma unroll
   for (int i = 0; i < 8; i++) acc[i] = 0;
-  for (int n = n0 + tr; n < n1; n += RPP) {
-    uint4 raw = *reinterpret_cast<const uint4*>(a.x + xbase + (int64_t)n * a.x_sn + tc * 8);
+  auto fold = [&](const uint4& raw) {
     const u16* e = reinterpret_cast<const u16*>(&raw);
 #pragma unroll
     for (int i = 0; i < 8; i++) {
@@ -209,7 +208,20 @@ __global__ void __launch_bounds__(256) colstat_partial_kernel(ColStatArgs a) {
       if constexpr (MODE == 0) acc[i] += (double)x;
       else acc[i] = fmaxf(acc[i], fabsf(x));
     }
+  };
+  // Eight independent 16-byte loads per lane in flight (the pass is a pure read: what limits it is the bytes on their
+  // way, not the arithmetic); the float64 sum of fp16/bf16 values is exact, so the order of the additions is free.
+  constexpr int UNR = 8;
+  const u16* base = a.x + xbase + tc * 8;
+  int n = n0 + tr;
+  for (; n + (UNR - 1) * RPP < n1; n += UNR * RPP) {
+    uint4 raw[UNR];
+#pragma unroll
+    for (int u = 0; u < UNR; u++) raw[u] = load_stream16(base + (int64_t)(n + u * RPP) * a.x_sn);
+#pragma unroll
+    for (int u = 0; u < UNR; u++) fold(raw[u]);
   }
+  for (; n < n1; n += RPP) fold(load_stream16(base + (int64_t)n * a.x_sn));
   __shared__ acc_t red[RPP][D];
 #pragma unroll
   for (int i = 0; i < 8; i++) red[tr][tc * 8 + i] = acc[i];
@@ -322,7 +334,7 @@ __device__ __forceinline__ void prep_v_tile(const PrepVArgs& a, const int pidx, 
     for (int j = 0; j < 4; j++) {
       const int r = n0 + 4 * quad + j;
       raw[j] = make_uint4(0, 0, 0, 0);
-      if (r < L) raw[j] = *reinterpret_cast<const uint4*>(a.v + vbase + (int64_t)r * a.v_sn + tc * 8);
+      if (r < L) raw[j] = load_stream16(a.v + vbase + (int64_t)r * a.v_sn + tc * 8);
     }
 #pragma unroll
     for (int i = 0; i < 8; i++) {
@@ -364,7 +376,7 @@ __device__ __forceinline__ void prep_v_tile(const PrepVArgs& a, const int pidx, 
       const uint32_t* src = &T[(32 * dt + d_lo) * TS + (4 * ks16 + hh) * 2];
       v = make_uint4(src[0], src[1], src[4], src[5]);
     }
-    out[c] = v;
+    store_stream16(out + c, v);
   }
 }
 
