@@ -44,6 +44,7 @@ SIGNATURES = {
     "sage_attn_fwd_masked": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I,
                                      _L, _L, _L, _L, _L, _L, _L, _L, _L, _I, _I, _I, _I, _P, _I, _L, _L, _L, _L, _P]),
     "sage_sageattn_workspace_bytes": (c_size_t, [_I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I]),
+    "sage_sageattn_workspace_bytes_for": (c_size_t, [_I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I]),
     "sage_sageattn": (c_int, [_P, _P, _P, _P, _P, _P, c_size_t, _I, _I, _I, _I, _I, _I,
                               _L, _L, _L, _L, _L, _L, _L, _L, _L, _L, _L, _L,
                               _I, _I, _I, c_double, _I, _I, _I, _P, _P, _I, _I, _P]),

@@ -16,6 +16,13 @@
  * wavefronts 4-7 vector instructions (valu_kind 0 v_fma_f32, 1 v_cvt_pk_u8_f32, 2 v_max3_i32, 3 a mix of the FP8
  * softmax with one conversion per code: 64 + 64 + 32 per iteration, 4 the mix the kernels run: 64 v_fma_f32 +
  * 32 v_cvt_pknorm_u16_f32 + 16 v_perm_b32 + 32 v_max3_i32).  mode 1 runs the MFMA half alone, 2 the vector half alone, 3 both.
+ *
+ * sage_period: the steady-state 128-key tile period of the FP8 P.V attention kernel at head_dim 128 as an instruction
+ * mix without the attention around it: eight wavefronts in two groups half a period apart, per wavefront and period 16
+ * INT8 MFMAs + 8 FP8 MFMAs + 2 row-sum MFMAs fed by 32 ds_read_b128, the 160-odd vector instructions of a tile's row
+ * maximum and probability codes, and four 1 KB global->LDS requests; one LDS-only barrier per period.  `parts` switches
+ * the pieces on (1 MFMAs, 2 fragments from LDS, 4 vector half, 8 requests).  What the schedule costs on the hardware
+ * before masks, rescales, prologue, epilogue and imbalance.
  */
 #ifndef SAGE_HW_RATES_H
 #define SAGE_HW_RATES_H
@@ -30,6 +37,7 @@ extern "C" {
 double sage_microbench_units(int kind);
 int sage_microbench(int kind, int grid, int waves_per_simd, int iters, void* sink, size_t sink_bytes, void* stream);
 int sage_coexec(int mfma_kind, int valu_kind, int mode, int grid, int iters, void* sink, size_t sink_bytes, void* stream);
+int sage_period(int parts, int grid, int periods, void* sink, size_t sink_bytes, const void* src, size_t src_bytes, void* stream);
 #ifdef __cplusplus
 }
 #endif

@@ -181,6 +181,179 @@ __global__ void __launch_bounds__(512) coexec_kernel(int* sink, int iters, int m
   sink[blockIdx.x * 1024 + threadIdx.x] = result;
 }
 
+// ---------------------------------------------------------------------------------------------
+// The steady-state tile period of the FP8 P.V attention kernel (head_dim 128, 128-key tiles) as an instruction mix
+// without the attention around it: a workgroup of eight wavefronts in two groups half a period apart, one LDS-only
+// barrier per period.  Per period every wavefront runs a matrix half -- P.V: 8 v_mfma_f32_32x32x64_f8f6f4 whose A
+// fragments are 16 ds_read_b128 (three pairs ahead) plus 2 v_mfma_f32_16x16x128_f8f6f4 on a resident operand; Q.K^T: 16
+// v_mfma_i32_32x32x32_i8 whose A fragments are 16 ds_read_b128 (four ahead), the first of each accumulator starting from
+// a resident bias block -- and a vector half on the 64 scores per lane the Q.K^T left: four integer max3 chains, the
+// exchange with the lane that shares the row, the block exponent and constants, 64 v_fma_f32, 32 v_cvt_pknorm_u16_f32,
+// 16 v_perm_b32, whose result is the B operand of the next P.V.  Group 0 issues four 1 KB global->LDS requests after its
+// matrix half, group 1 four at the start of its period (32 KB per period and workgroup, from a 1 MB window per
+// XCD -- workgroup index modulo 8 -- that its L2 serves after the first pass, as the shared K/V tiles of a head are).  PARTS switches the pieces on: 1 MFMAs, 2 fragment reads from LDS
+// (off: the MFMAs take resident registers), 4 the vector half, 8 the global->LDS requests.  The time of a period with
+// everything on is what this schedule costs on the hardware before any attention-specific overhead (masks, rescales,
+// prologue, epilogue, imbalance); with single pieces on, what each of them costs alone.
+// ---------------------------------------------------------------------------------------------
+template <int PARTS>
+__global__ void __launch_bounds__(512) period_kernel(int* sink, const uint8_t* src, int periods, float s, float c) {
+  constexpr bool MFMA = PARTS & 1, LDSF = PARTS & 2, VEC = PARTS & 4, DMA = PARTS & 8;
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];   // 64 KB of fragments + 32 KB that the requests fill
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63, grp = wave >> 2;
+  for (int i = threadIdx.x; i < 65536 / 4; i += 512) reinterpret_cast<int*>(smem)[i] = i * 7 + 1;
+  __syncthreads();
+  const __amdgpu_buffer_rsrc_t rsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void*)(src + (size_t)(blockIdx.x & 7) * (1u << 20)), 0, 0x7fffffff, 0x00020000);
+  v4i q[4];
+  v16i bias, acc[4];
+  v16f o[4];
+  v4f osum = {0.f, 0.f, 0.f, 0.f};
+  v8i ones;
+  for (int k = 0; k < 4; k++) q[k] = v4i{lane + k, 1, 2, 3};
+  for (int i = 0; i < 16; i++) bias[i] = 0x4B400000;
+  for (int i = 0; i < 8; i++) ones[i] = (lane == 0 || lane == 32 || lane == 20 || lane == 52) ? 0x38383838 : 0;
+  for (int k = 0; k < 4; k++) { acc[k] = bias; for (int i = 0; i < 16; i++) o[k][i] = 0.f; }
+  asm volatile("" : "+v"(bias), "+v"(ones));
+  float m_used = 0.f, lsum = 0.f, sc = s * 1e-4f;
+  int pscale = 119;
+  auto matrix_half = [&](int p) {
+    if constexpr (!MFMA) return;
+    const uint8_t* vbuf = smem + ((p & 1) ? 32768 : 0) + lane * 16;
+    const uint8_t* kbuf = smem + ((p & 1) ? 0 : 32768) + 16384 + lane * 16;
+    {   // P.V: the packed probabilities are registers 0..15 of acc[0]
+      v8i vf[8];
+      auto vfrag = [&](int i) {
+        if constexpr (!LDSF) return v8i{acc[1][0], 1, 2, 3, 4, 5, 6, i};
+        const v4i lo = *reinterpret_cast<const v4i*>(vbuf + (2 * i) * 1024), hi = *reinterpret_cast<const v4i*>(vbuf + (2 * i + 1) * 1024);
+        return v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      };
+#pragma unroll
+      for (int i = 0; i < 3; i++) vf[i] = vfrag(i);
+#pragma unroll
+      for (int i = 0; i < 8; i++) {
+        const int kk = i / 4, dt = i % 4;
+        if (i + 3 < 8) vf[i + 3] = vfrag(i + 3);
+        v8i pb;
+#pragma unroll
+        for (int e = 0; e < 8; e++) pb[e] = acc[0][8 * kk + e];
+        if (dt == 0) {
+          const v4f zero = {0.f, 0.f, 0.f, 0.f};
+          osum = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ones, pb, kk == 0 ? zero : osum, 0, 0, 0, 0, 0, 0);
+        }
+        o[dt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vf[i], pb, o[dt], 0, 0, 0, 127, 0, pscale);
+      }
+      if constexpr (LDSF) {
+        __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+          if (i % 4 == 0) __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          if (i + 3 < 8) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        }
+      }
+    }
+    {   // Q.K^T
+      v4i kf[16];
+      auto kfrag = [&](int i) {
+        if constexpr (!LDSF) return v4i{(int)o[0][0], 1, 2, i};
+        return *reinterpret_cast<const v4i*>(kbuf + i * 1024);
+      };
+#pragma unroll
+      for (int i = 0; i < 4; i++) kf[i] = kfrag(i);
+#pragma unroll
+      for (int i = 0; i < 16; i++) {
+        if (i + 4 < 16) kf[i + 4] = kfrag(i + 4);
+        const int nt = i % 4, ks = i / 4;
+        acc[nt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf[i], q[ks], ks == 0 ? bias : acc[nt], 0, 0, 0);
+      }
+      if constexpr (LDSF) {
+        __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+#pragma unroll
+        for (int i = 0; i < 12; i++) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+      }
+    }
+  };
+  auto vector_half = [&]() {
+    if constexpr (!VEC) return;
+    int mxg[4];
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+      mxg[t] = acc[t][0];
+#pragma unroll
+      for (int r = 1; r < 16; r++) mxg[t] = max(mxg[t], acc[t][r]);
+    }
+    const int mx = max(max(mxg[0], mxg[1]), max(mxg[2], mxg[3]));
+    float mloc = __builtin_fmaf(__builtin_bit_cast(float, mx), sc, -12582912.0f * sc);
+    auto r2 = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(int, mloc), __builtin_bit_cast(int, mloc), false, false);
+    const float mall = fmaxf(__builtin_bit_cast(float, (int)r2[0]), __builtin_bit_cast(float, (int)r2[1]));
+    lsum = __builtin_fmaf(osum[0], __builtin_bit_cast(float, pscale << 23), lsum);
+    if (__builtin_amdgcn_ballot_w64(mall > m_used + 1.0e30f) != 0) m_used = mall;      // (never taken: the rescale is rare)
+    const float e = fmaxf(__builtin_ceilf(mall - m_used), -110.0f);
+    constexpr float kN8 = 8.0f * 256.0f / 65535.0f;
+    const float k0 = __builtin_fmaf(-kN8, e, __builtin_fmaf(kN8, 8.75f - m_used, c));
+    pscale = (int)(unsigned)(e + 119.0f);
+    const float mul = kN8 * sc, cc = __builtin_fmaf(-12582912.0f, mul, k0);
+#pragma unroll
+    for (int nt = 0; nt < 4; nt++) {
+      float t8[16];
+#pragma unroll
+      for (int r = 0; r < 16; r++) t8[r] = __builtin_fmaf(__builtin_bit_cast(float, (int)acc[nt][r]), mul, cc);
+#pragma unroll
+      for (int q4 = 0; q4 < 4; q4++) {
+        const unsigned w01 = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_pknorm_u16(t8[4 * q4], t8[4 * q4 + 1]));
+        const unsigned w23 = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_pknorm_u16(t8[4 * q4 + 2], t8[4 * q4 + 3]));
+        acc[0][4 * nt + q4] = (int)__builtin_amdgcn_perm(w23, w01, 0x07050301u);
+      }
+    }
+    sc = sc * 1.0000001f;
+  };
+  auto requests = [&](int p) {
+    if constexpr (!DMA) return;
+    uint8_t* dst = smem + 65536 + (wave & 3) * 8192 + grp * 4096;       // (the data is never read: only the traffic matters)
+    const int uo = ((p * 32768) & ((1 << 20) - 1)) + wave * 4096;
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)(dst + i * 1024), 16, lane * 16, uo + i * 1024, 0, 0);
+  };
+  auto period_start = [&]() {
+    if constexpr (DMA) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");     // the requests of the period before last have landed
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    if constexpr (!MFMA) {      // without the MFMAs nothing renews the scores: keep the vector half from being hoisted
+#pragma unroll
+      for (int k = 0; k < 4; k++) asm volatile("" : "+v"(acc[k]));
+    }
+  };
+  // (one loop per group, as in the attention kernel: two copies of the matrix half inside one loop cost the compiler its
+  // register allocation)
+  if (grp == 0) {
+    for (int p = 0; p < periods; p++) { period_start(); matrix_half(p); requests(p); vector_half(); }
+  } else {
+    for (int p = 0; p < periods; p++) { period_start(); requests(p); vector_half(); matrix_half(p); }
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  int result = (int)lsum ^ pscale;
+  for (int k = 0; k < 4; k++) result ^= acc[k][0] ^ (int)o[k][0];
+  sink[blockIdx.x * 1024 + threadIdx.x] = result;
+}
+
+template <int PARTS>
+hipError_t launch_period(int* sink, const uint8_t* src, int grid, int periods, hipStream_t st) {
+  auto kern = period_kernel<PARTS>;
+  static bool attr_done = false;
+  if (!attr_done) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 98304);
+    if (e != hipSuccess) return e;
+    attr_done = true;
+  }
+  kern<<<dim3(grid), dim3(512), 98304, st>>>(sink, src, periods, 0.999f, 0.001f);
+  return hipGetLastError();
+}
+
 template <int MK, int VK>
 hipError_t launch_coexec(int* sink, int grid, int iters, int mode, hipStream_t st) {
   coexec_kernel<MK, VK><<<dim3(grid), dim3(512), 0, st>>>(sink, iters, mode, 0.999f, 0.001f);
@@ -241,6 +414,31 @@ int sage_microbench(int kind, int grid, int waves_per_simd, int iters, void* sin
 // Co-execution benchmark: `grid` workgroups of eight wavefronts, `iters` iterations; mfma_kind 0 (INT8) or 1 (FP8),
 // valu_kind 0 fma, 1 cvt_pk_u8, 2 max3, 3 the mix with one conversion per code, 4 the mix with two per conversion; mode 1 = the MFMA wavefronts only, 2 = the vector wavefronts only,
 // 3 = both.  Per iteration a wavefront issues 16 MFMAs, or 64 / 64 / 32 / 160 / 144 vector instructions.
+// The attention kernel's steady-state tile period as an instruction mix (see period_kernel): `parts` is a sum of 1 (MFMAs),
+// 2 (their A fragments come from LDS), 4 (the vector half), 8 (the global->LDS tile requests); supported: 1, 3, 4, 5, 7,
+// 11, 15.  `src` is device memory of at least grid MiB that the requests read.  The caller times the launch and divides
+// by `periods`.
+int sage_period(int parts, int grid, int periods, void* sink, size_t sink_bytes, const void* src, size_t src_bytes, void* stream) {
+  using namespace sage;
+  if (grid <= 0 || grid > 65535 || periods <= 0 || !sink || !src) return HWR_EINVAL;
+  if (sink_bytes < (size_t)grid * 1024 * sizeof(int) || src_bytes < (size_t)grid << 20) return HWR_ESIZE;
+  int* out = (int*)sink;
+  const uint8_t* in = (const uint8_t*)src;
+  hipStream_t st = (hipStream_t)stream;
+  hipError_t e;
+  switch (parts) {
+    case 1: e = launch_period<1>(out, in, grid, periods, st); break;
+    case 3: e = launch_period<3>(out, in, grid, periods, st); break;
+    case 4: e = launch_period<4>(out, in, grid, periods, st); break;
+    case 5: e = launch_period<5>(out, in, grid, periods, st); break;
+    case 7: e = launch_period<7>(out, in, grid, periods, st); break;
+    case 11: e = launch_period<11>(out, in, grid, periods, st); break;
+    case 15: e = launch_period<15>(out, in, grid, periods, st); break;
+    default: return HWR_EINVAL;
+  }
+  return e == hipSuccess ? HWR_OK : HWR_ELAUNCH;
+}
+
 int sage_coexec(int mfma_kind, int valu_kind, int mode, int grid, int iters, void* sink, size_t sink_bytes, void* stream) {
   using namespace sage;
   if (mfma_kind < 0 || mfma_kind > 1 || valu_kind < 0 || valu_kind > 4 || mode < 1 || mode > 3) return HWR_EINVAL;

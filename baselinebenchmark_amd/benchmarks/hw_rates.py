@@ -33,6 +33,8 @@ def lib() -> ctypes.CDLL:
         h.sage_microbench.argtypes = [ctypes.c_int] * 4 + [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
         h.sage_coexec.restype = ctypes.c_int
         h.sage_coexec.argtypes = [ctypes.c_int] * 5 + [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
+        h.sage_period.restype = ctypes.c_int
+        h.sage_period.argtypes = [ctypes.c_int] * 3 + [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
         _lib = h
     return _lib
 
@@ -128,14 +130,52 @@ def run_coexec(iters: int = 20000) -> list[dict]:
     return rows
 
 
+PERIOD_PARTS = [
+    (1, "MFMAs only, operands in registers"),
+    (3, "MFMAs with their A fragments from LDS"),
+    (11, "... and the global->LDS tile requests"),
+    (4, "vector half only"),
+    (5, "MFMAs (registers) + vector half"),
+    (7, "MFMAs from LDS + vector half"),
+    (15, "everything: the kernel's period"),
+]
+
+
+def run_period(periods: int = 4000) -> list[dict]:
+    """The attention kernel's steady-state tile period as an instruction mix (hw_rates.hip: period_kernel), one
+    workgroup per compute unit, wall clock per period, for the pieces alone and together."""
+    n_cu = torch.cuda.get_device_properties(0).multi_processor_count
+    sink = torch.empty(n_cu * 1024, dtype=torch.int32, device="cuda")
+    src = torch.zeros(n_cu << 20, dtype=torch.uint8, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    rows = []
+    for parts, name in PERIOD_PARTS:
+        def launch():
+            check(lib().sage_period(parts, n_cu, periods, sink.data_ptr(), sink.numel() * 4, src.data_ptr(), src.numel(), stream))
+        launch()
+        torch.cuda.synchronize()
+        best = float("inf")
+        for _ in range(3):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(); launch(); e1.record()
+            torch.cuda.synchronize()
+            best = min(best, e0.elapsed_time(e1) * 1e-3)
+        ns = best / periods * 1e9
+        # a period computes 256 query rows x 128 keys x head_dim 128 of both products
+        rows.append({"parts": parts, "name": name, "ns_per_period": ns,
+                     "chip_TOPS_if_the_whole_kernel_ran_like_this": 4.0 * 256 * 128 * 128 * n_cu / ns / 1e3})
+    return rows
+
+
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(description=__doc__)
     ap.add_argument("--json", action="store_true", help="print one JSON document instead of the table")
     args = ap.parse_args(argv)
     rows = run()
     co = run_coexec()
+    per = run_period()
     if args.json:
-        print(json.dumps({"rates": rows, "coexecution": co}))
+        print(json.dumps({"rates": rows, "coexecution": co, "period": per}))
         return 0
     print(f"{'benchmark':58s} waves/SIMD  result")
     for r in rows:
@@ -152,6 +192,11 @@ def main(argv=None) -> int:
         print(f"{r['mfma']:34s} + {r['valu']:46s} alone {r['mfma_alone_s'] * 1e3:6.3f} / {r['valu_alone_s'] * 1e3:6.3f} ms "
               f"({r['ns_per_mfma']:.1f} ns per MFMA, {r['ns_per_valu_instruction']:.2f} ns per vector instruction), both "
               f"{r['both_s'] * 1e3:6.3f} ms, overlap {100 * r['overlap']:.0f} %")
+    print("\nthe attention kernel's tile period (FP8 P.V, head_dim 128, 128 keys, eight wavefronts in two groups) as an instruction mix;"
+          " 2176 matrix-pipe cycles per SIMD = 0.91 us at 2.4 GHz")
+    for r in per:
+        print(f"{r['name']:48s} {r['ns_per_period']:7.1f} ns per period   {r['chip_TOPS_if_the_whole_kernel_ran_like_this']:6.0f} TOPS "
+              f"({100 * r['chip_TOPS_if_the_whole_kernel_ran_like_this'] / 5033.2:.0f} % of peak) if a kernel were nothing but this")
     return 0
 
 

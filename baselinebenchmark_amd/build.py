@@ -83,7 +83,9 @@ def build_tools(verbose: bool = True) -> list[Path]:
     library (tile_timing), the hardware-rate micro-benchmarks (hw_rates) and the C++ benchmark driver."""
     out = [build(verbose, timing=True)]
     obj = BENCH / "hw_rates.o"
-    res = subprocess.run([_hipcc(), *FLAGS, "-c", str(BENCH / "hw_rates.hip"), "-o", str(obj)], capture_output=True, text=True)
+    # (the attention kernels' scheduling flags: the micro-benchmarks reproduce their instruction streams)
+    res = subprocess.run([_hipcc(), *FLAGS, *EXTRA_FLAGS["sage_attn.hip"], "-c", str(BENCH / "hw_rates.hip"), "-o", str(obj)],
+                         capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError(f"hipcc failed for hw_rates.hip:\n{res.stderr}")
     out.append(_link([obj], HWRATES_LIB, verbose))

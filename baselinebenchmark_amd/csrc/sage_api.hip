@@ -341,21 +341,27 @@ struct E2EWorkspace {
   size_t q_i8, k_i8, q_scale, k_scale, km, v_scale, panels, stat, plan, lse_off, total;
   int64_t qs_sh, ks_sh, panel_sh;
 };
+// What a call needs beyond K, V and their statistics: the INT8 copy of Q with its scales (only when Q is quantised by the
+// stand-alone pass: an explicit mask, the LSE correction of K smoothing, interleaved Q scales) and the per-row LSE
+// correction term (only when LSE is returned from smoothed keys).
+bool needs_q_pass(int blkq, int has_mask, int want_lse, int smooth_k) {
+  return has_mask || (want_lse && smooth_k) || blk_groups(blkq) != 1;
+}
 E2EWorkspace e2e_layout(int B, int Hq, int Hkv, int Sq, int Skv, int D, int blkq, int blkk, int pv, int total_q, int total_k,
-                        int varlen) {
+                        int varlen, bool q_pass, bool lse_offset) {
   E2EWorkspace w;
   size_t off = 0;
   size_t nq = varlen ? (size_t)total_q * Hq * D : (size_t)B * Hq * Sq * D;
   size_t nk = varlen ? (size_t)total_k * Hkv * D : (size_t)B * Hkv * Skv * D;
-  w.q_i8 = off; off += align_up(nq);
+  w.q_i8 = off; off += q_pass ? align_up(nq) : 0;
   w.k_i8 = off; off += align_up(nk);
   if (varlen) {
     w.qs_sh = total_q / blk_rows(blkq) + B; w.ks_sh = total_k / blk_rows(blkk) + B; w.panel_sh = total_k / SAGE_PANEL_ROWS + B;
-    w.q_scale = off; off += align_up((size_t)Hq * w.qs_sh * 4);
+    w.q_scale = off; off += q_pass ? align_up((size_t)Hq * w.qs_sh * 4) : 0;
     w.k_scale = off; off += align_up((size_t)Hkv * w.ks_sh * 4);
   } else {
     w.qs_sh = w.ks_sh = w.panel_sh = 0;
-    w.q_scale = off; off += align_up((size_t)B * Hq * ((Sq + blk_rows(blkq) - 1) / blk_rows(blkq)) * blk_groups(blkq) * 4);
+    w.q_scale = off; off += q_pass ? align_up((size_t)B * Hq * ((Sq + blk_rows(blkq) - 1) / blk_rows(blkq)) * blk_groups(blkq) * 4) : 0;
     w.k_scale = off; off += align_up((size_t)B * Hkv * ((Skv + blk_rows(blkk) - 1) / blk_rows(blkk)) * (blk_groups(blkk) ? blk_groups(blkk) : 1) * 4);
   }
   w.km = off; off += align_up((size_t)B * Hkv * D * 2);
@@ -366,7 +372,7 @@ E2EWorkspace e2e_layout(int B, int Hq, int Hkv, int Sq, int Skv, int D, int blkq
   size_t stat2 = sage_prep_v_workspace_bytes(B, Hkv, Skv, D, pv);
   w.stat = off; off += align_up(stat > stat2 ? stat : stat2);
   w.plan = off; off += varlen ? align_up(sage_varlen_plan_ints(B, total_q) * 4) : 0;
-  w.lse_off = off; off += align_up((varlen ? (size_t)Hq * total_q : (size_t)B * Hq * Sq) * 4);
+  w.lse_off = off; off += lse_offset ? align_up((varlen ? (size_t)Hq * total_q : (size_t)B * Hq * Sq) * 4) : 0;
   w.total = off;
   return w;
 }
@@ -375,7 +381,14 @@ E2EWorkspace e2e_layout(int B, int Hq, int Hkv, int Sq, int Skv, int D, int blkq
 size_t sage_sageattn_workspace_bytes(int B, int Hq, int Hkv, int Sq, int Skv, int D, int blkq, int blkk, int pv_mode,
                                      int total_q, int total_k, int varlen) {
   if (blkq <= 0 || blkk <= 0) return 0;
-  return e2e_layout(B, Hq, Hkv, Sq, Skv, D, blkq, blkk, pv_mode, total_q, total_k, varlen).total;
+  return e2e_layout(B, Hq, Hkv, Sq, Skv, D, blkq, blkk, pv_mode, total_q, total_k, varlen, true, true).total;
+}
+
+size_t sage_sageattn_workspace_bytes_for(int B, int Hq, int Hkv, int Sq, int Skv, int D, int blkq, int blkk, int pv_mode,
+                                         int total_q, int total_k, int varlen, int smooth_k, int want_lse, int has_mask) {
+  if (blkq <= 0 || blkk <= 0) return 0;
+  return e2e_layout(B, Hq, Hkv, Sq, Skv, D, blkq, blkk, pv_mode, total_q, total_k, varlen,
+                    needs_q_pass(blkq, has_mask, want_lse, smooth_k), want_lse && smooth_k).total;
 }
 
 int sage_sageattn(const void* q, const void* k, const void* v, void* out, float* lse, void* workspace, size_t workspace_bytes,
@@ -409,7 +422,11 @@ int sage_sageattn_masked(const void* q, const void* k, const void* v, void* out,
   if (varlen && !cu_seqlens_k) return fail(SAGE_EINVAL, "packed mode needs cu_seqlens_k");
   if (B == 0 || Hq == 0 || Sq == 0) return SAGE_OK;
   if (!workspace) return fail(SAGE_EWORKSPACE, "null workspace");
-  E2EWorkspace w = e2e_layout(B, Hq, Hkv, Sq, Skv, D, blkq, blkk, pv_mode, total_q, total_k, varlen);
+  // (the workspace is laid out for what THIS call uses; sage_sageattn_workspace_bytes is the upper bound over all calls
+  // of the shape, sage_sageattn_workspace_bytes_for the size for one kind of call)
+  const bool q_pass = needs_q_pass(blkq, attn_mask != nullptr, lse != nullptr, smooth_k && !(!varlen && Skv == 0));
+  E2EWorkspace w = e2e_layout(B, Hq, Hkv, Sq, Skv, D, blkq, blkk, pv_mode, total_q, total_k, varlen, q_pass,
+                              lse != nullptr && smooth_k && !(!varlen && Skv == 0));
   if (workspace_bytes < w.total) return fail(SAGE_EWORKSPACE, "workspace too small: %zu < %zu", workspace_bytes, w.total);
   if (reinterpret_cast<uintptr_t>(workspace) % 256) return fail(SAGE_EINVAL, "workspace must be 256-byte aligned");
   uint8_t* ws = (uint8_t*)workspace;

@@ -58,8 +58,8 @@ int sage_sageattn_static(const void* q, const void* k, const void* v, void* out,
                          sage_stream_t stream) {
   if (blkq <= 0 || blkk <= 0 || B < 0 || Hq < 0 || Hkv <= 0 || Sq < 0 || Skv < 0 || D <= 0 || total_q < 0 || total_k < 0)
     return sage::set_error(SAGE_EINVAL, "sage_sageattn_static: bad dimension or block size");
-  const size_t need = sage_sageattn_workspace_bytes(B, Hq, Hkv, Sq, Skv, D, blkq, blkk, pv_mode, total_q, total_k,
-                                                    cu_seqlens_q != nullptr);
+  const size_t need = sage_sageattn_workspace_bytes_for(B, Hq, Hkv, Sq, Skv, D, blkq, blkk, pv_mode, total_q, total_k,
+                                                        cu_seqlens_q != nullptr, smooth_k, lse != nullptr, 0);
   if (need > (size_t)SAGE_STATIC_SCRATCH_BYTES) {
     char msg[256];
     snprintf(msg, sizeof(msg),

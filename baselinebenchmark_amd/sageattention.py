@@ -431,7 +431,8 @@ def sageattn(q, k, v, tensor_layout="HND", is_causal=False, sm_scale=None, smoot
     out = torch.empty(q.shape, device=q.device, dtype=q.dtype)
     _, _, _, _, osb, osh, osn = _layout(out, tensor_layout)
     lse = torch.empty((B, Hq, Sq), device=q.device, dtype=torch.float32) if return_lse else None
-    ws_bytes = lib().sage_sageattn_workspace_bytes(B, Hq, Hkv, Sq, Skv, D, BLKQ | qflag, BLKK | kflag, pv, 0, 0, 0)
+    ws_bytes = lib().sage_sageattn_workspace_bytes_for(B, Hq, Hkv, Sq, Skv, D, BLKQ | qflag, BLKK | kflag, pv, 0, 0, 0,
+                                                       int(bool(smooth_k)), int(bool(return_lse)), int(attn_mask is not None))
     ws = torch.empty(max(ws_bytes, 256), device=q.device, dtype=torch.uint8)
     if attn_mask is not None:
         if is_causal:
@@ -500,8 +501,8 @@ def sageattn_varlen(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqle
     pv = _pv(pv_mode)
     out = torch.empty_like(q)
     lse = torch.empty((Hq, Tq), device=q.device, dtype=torch.float32) if return_lse else None
-    ws_bytes = lib().sage_sageattn_workspace_bytes(nseq, Hq, Hkv, int(max_seqlen_q), int(max_seqlen_k), D, BLKQ, BLKK, pv,
-                                                   Tq, Tk, 1)
+    ws_bytes = lib().sage_sageattn_workspace_bytes_for(nseq, Hq, Hkv, int(max_seqlen_q), int(max_seqlen_k), D, BLKQ, BLKK, pv,
+                                                       Tq, Tk, 1, int(bool(smooth_k)), int(bool(return_lse)), 0)
     ws = torch.empty(max(ws_bytes, 256), device=q.device, dtype=torch.uint8)
     check(lib().sage_sageattn(_ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _ptr(ws), ws_bytes,
                               nseq, Hq, Hkv, int(max_seqlen_q), int(max_seqlen_k), D,

@@ -236,6 +236,14 @@ int sage_attn_fwd_masked(const int8_t* q, const int8_t* k, const void* v_panels,
 size_t sage_sageattn_workspace_bytes(int B, int Hq, int Hkv, int Sq, int Skv, int D,
                                      int blkq, int blkk, int pv_mode, int total_q, int total_k,
                                      int varlen);
+/* The same for ONE kind of call: without an explicit mask, and unless LSE is returned from smoothed keys or the Q scales
+ * are interleaved, Q is quantised inside the attention kernel and its INT8 copy (a third of the upper bound) is not
+ * part of the workspace.  sage_sageattn / sage_sageattn_masked accept any workspace of at least this size for the call
+ * they are given; sage_sageattn_static checks it against its capacity. */
+size_t sage_sageattn_workspace_bytes_for(int B, int Hq, int Hkv, int Sq, int Skv, int D,
+                                         int blkq, int blkk, int pv_mode,
+                                         int total_q, int total_k, int varlen,
+                                         int smooth_k, int want_lse, int has_mask);
 int sage_sageattn(const void* q, const void* k, const void* v, void* out, float* lse,
                   void* workspace, size_t workspace_bytes,
                   int B, int Hq, int Hkv, int Sq, int Skv, int D,
@@ -277,7 +285,10 @@ int sage_sageattn_masked(const void* q, const void* k, const void* v, void* out,
  * scales, K mean, V panels, statistics partials, the packed-batch plan, INT8 Q where a separate pass is needed)
  * live in an array of SAGE_STATIC_SCRATCH_BYTES that is part of the library's device image, one copy per GPU,
  * held until the process ends.  The call allocates and frees nothing and does not synchronise.
- * Limit: sage_sageattn_workspace_bytes(...) of the problem must not exceed sage_sageattn_static_capacity()
+ * The FIRST call on a device (of this entry point, and of each kernel variant it launches) additionally looks up the
+ * array's address and raises the kernels' dynamic-LDS limit -- runtime calls that may allocate and are not allowed
+ * while a stream is capturing: make one call of the same kind outside the capture first (tests/test_zz_no_alloc.py).
+ * Limit: sage_sageattn_workspace_bytes_for(...) of the call must not exceed sage_sageattn_static_capacity()
  * (= SAGE_STATIC_SCRATCH_BYTES); larger problems return SAGE_EWORKSPACE and launch nothing.
  * All calls on one GPU share that GPU's array: calls that may overlap on one GPU (different streams, or host
  * threads without ordering between their streams) race; serialise them or use sage_sageattn.  The array keeps

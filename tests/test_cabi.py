@@ -40,6 +40,18 @@ def test_size_queries_do_not_need_a_gpu(sage_lib):
     assert sage_lib.sage_k_mean_workspace_bytes(2, 32, 16384, 128) >= 2 * 32 * 32 * 128 * 8
     assert sage_lib.sage_sageattn_workspace_bytes(2, 32, 32, 16384, 16384, 128, 64, 128, 1, 0, 0, 0) > 3 * 2 * 32 * 16384 * 128
     # eight interleaved Q scales per block: seven more floats per (batch, head, block)
+    # by need: the INT8 copy of Q (B*Hq*Sq*D bytes) and the LSE correction term are only part of a call that uses them
+    c2 = (2, 32, 32, 16384, 16384, 128, 64, 128, 1, 0, 0, 0)
+    bound = sage_lib.sage_sageattn_workspace_bytes(*c2)
+    plain = sage_lib.sage_sageattn_workspace_bytes_for(*c2, 1, 0, 0)
+    with_lse = sage_lib.sage_sageattn_workspace_bytes_for(*c2, 1, 1, 0)
+    lse_unsmoothed = sage_lib.sage_sageattn_workspace_bytes_for(*c2, 0, 1, 0)
+    masked = sage_lib.sage_sageattn_workspace_bytes_for(*c2, 1, 0, 1)
+    nq = 2 * 32 * 16384 * 128
+    assert bound == with_lse >= masked > plain == lse_unsmoothed
+    assert bound - plain >= nq + 2 * 32 * 16384 * 4 and plain < bound - nq
+    assert sage_lib.sage_sageattn_workspace_bytes_for(1, 4, 4, 4096, 4096, 128, 32 | 0x100, 64, 1, 0, 0, 0, 1, 0, 0) > \
+        sage_lib.sage_sageattn_workspace_bytes_for(1, 4, 4, 4096, 4096, 128, 32, 64, 1, 0, 0, 0, 1, 0, 0) + 4 * 4096 * 128 - 1
     a = sage_lib.sage_sageattn_workspace_bytes(1, 4, 4, 4096, 4096, 128, 32, 64, 1, 0, 0, 0)
     b = sage_lib.sage_sageattn_workspace_bytes(1, 4, 4, 4096, 4096, 128, 32 | 0x100, 64, 1, 0, 0, 0)
     assert b - a == 4 * 128 * 7 * 4

@@ -236,7 +236,10 @@ def test_lse_is_empty_unless_requested():
                                  ("NHD", 2, 4, 2, 300, 1000, 128, torch.bfloat16, 64, 64),
                                  ("HND", 1, 2, 1, 129, 1024, 128, torch.bfloat16, 32, 16),
                                  ("HND", 1, 2, 1, 40, 1025, 128, torch.bfloat16, 64, 128),     # one key too many: the six-launch path
-                                 ("HND", 3, 2, 2, 77, 513, 64, torch.float16, 128, 32)])
+                                 ("HND", 3, 2, 2, 77, 513, 64, torch.float16, 128, 32),
+                                 # the dearest case of the short path: 64 (batch, head) pairs x 64 K tiles of 16 keys at
+                                 # head_dim 64, exactly 4 M elements of K, every tile re-reading its whole sequence
+                                 ("HND", 8, 8, 8, 64, 1024, 64, torch.bfloat16, 64, 16)])
 def test_one_call_on_short_sequences_equals_the_separate_calls_bitwise(cfg, pv, smooth):
     """Up to 1024 keys (and 4 M elements of K) the one-call pipeline runs its K and V pre-passes as ONE launch, whose workgroups compute the K
     mean / V scale of their sequence themselves; the separate entry points use the two-stage statistics kernels.  Same

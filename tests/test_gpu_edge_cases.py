@@ -115,7 +115,9 @@ def test_strided_views_of_a_fused_qkv_buffer_through_the_c_abi(pv, causal, lse):
     assert not q.is_contiguous()
     obuf = torch.zeros((B, S, 2, H, D), dtype=torch.bfloat16, device=DEV)
     out = obuf[:, :, 1]
-    need = _cabi.lib().sage_sageattn_workspace_bytes(B, H, H, S, S, D, 64, 128, _cabi.PV_FP8 if pv == "fp8" else _cabi.PV_FP16, 0, 0, 0)
+    need = _cabi.lib().sage_sageattn_workspace_bytes_for(B, H, H, S, S, D, 64, 128, _cabi.PV_FP8 if pv == "fp8" else _cabi.PV_FP16,
+                                                         0, 0, 0, 1, int(lse), 0)   # exactly what THIS call uses
+    assert need <= _cabi.lib().sage_sageattn_workspace_bytes(B, H, H, S, S, D, 64, 128, _cabi.PV_FP8 if pv == "fp8" else _cabi.PV_FP16, 0, 0, 0)
     guard = 1 << 16
     buf = torch.full((need + 2 * guard + 256,), 0x5A, dtype=torch.uint8, device=DEV)
     base = (-(buf.data_ptr() + guard)) % 256 + guard

@@ -66,6 +66,51 @@ def test_static_entry_point_lse_and_packed_batch():
     assert torch.equal(got.view(torch.int16), ref.view(torch.int16))
 
 
+def test_static_entry_point_takes_what_fits_without_the_int8_copy_of_q():
+    """The limit is checked against what the call uses: without LSE or a mask Q is quantised inside the attention kernel,
+    so a problem whose upper-bound workspace (with the INT8 copy of Q) exceeds the array still fits."""
+    lib = _cabi.lib()
+    B, H, S, D = 1, 24, 8192, 128
+    args = (B, H, H, S, S, D, 64, 128, _cabi.PV_FP8, 0, 0, 0)
+    assert lib.sage_sageattn_workspace_bytes(*args) > lib.sage_sageattn_static_capacity() >= lib.sage_sageattn_workspace_bytes_for(*args, 1, 0, 0)
+    q, k, v = _pair(B, H, S, D, torch.bfloat16, 123)
+    ref, got = torch.empty_like(q), torch.full_like(q, float("nan"))
+    assert sageattn_cabi(q, k, v, ref, is_causal=True, pv="fp8", BLKQ=64, BLKK=128) == 0
+    assert sageattn_cabi(q, k, v, got, is_causal=True, pv="fp8", BLKQ=64, BLKK=128, static=True) == 0, lib.sage_last_error().decode()
+    torch.cuda.synchronize()
+    assert torch.equal(got.view(torch.int16), ref.view(torch.int16))
+    # with LSE from smoothed keys the stand-alone Q pass and its INT8 copy come back: too large for the array
+    lse = torch.empty((B, H, S), device=DEV, dtype=torch.float32)
+    assert sageattn_cabi(q, k, v, got, is_causal=True, pv="fp8", BLKQ=64, BLKK=128, static=True, lse=lse) == _cabi.SAGE_EWORKSPACE
+
+
+def test_static_entry_point_under_graph_capture():
+    """The use the entry point is for.  The first call on a device looks up the array's address and sets kernel
+    attributes -- runtime calls that do not belong inside a capture -- so one warm-up call is made outside; the captured
+    call then only launches kernels.  Every replay must reproduce the eager result bit for bit (the program's own eager
+    work and synchronisations in between)."""
+    q, k, v = _pair(1, 4, 1200, 128, torch.bfloat16, 31)
+    ref, got = torch.empty_like(q), torch.full_like(q, float("nan"))
+    assert sageattn_cabi(q, k, v, ref, is_causal=True, pv="fp8", BLKQ=64, BLKK=128, static=True) == 0      # warm-up, outside
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            rc = sageattn_cabi(q, k, v, got, is_causal=True, pv="fp8", BLKQ=64, BLKK=128, static=True)
+    assert rc == 0, _cabi.lib().sage_last_error().decode()
+    for replay in range(3):
+        got.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(got.view(torch.int16), ref.view(torch.int16)), replay
+        # eager work between the replays, on the same array
+        other = torch.empty_like(q)
+        assert sageattn_cabi(q, k * 2, v, other, is_causal=False, pv="fp16", BLKQ=64, BLKK=128, static=True) == 0
+        torch.cuda.synchronize()
+
+
 def test_static_entry_point_rejects_what_does_not_fit():
     lib = _cabi.lib()
     cap = lib.sage_sageattn_static_capacity()
