@@ -21,8 +21,10 @@
  * mix without the attention around it: eight wavefronts in two groups half a period apart, per wavefront and period 16
  * INT8 MFMAs + 8 FP8 MFMAs + 2 row-sum MFMAs fed by 32 ds_read_b128, the 160-odd vector instructions of a tile's row
  * maximum and probability codes, and four 1 KB global->LDS requests; one LDS-only barrier per period.  `parts` switches
- * the pieces on (1 MFMAs, 2 fragments from LDS, 4 vector half, 8 requests).  What the schedule costs on the hardware
- * before masks, rescales, prologue, epilogue and imbalance.
+ * the pieces on (1 MFMAs, 2 fragments from LDS, 4 vector half, 8 requests); `random_operands` chooses the operand bits
+ * (0 a regular low-entropy pattern, 1 hashed bytes: the same instructions, but the multipliers, the register file and
+ * LDS see bits that toggle, and the clock the part sustains differs).  What the schedule costs on the hardware before
+ * masks, rescales, prologue, epilogue and imbalance.
  */
 #ifndef SAGE_HW_RATES_H
 #define SAGE_HW_RATES_H
@@ -37,7 +39,7 @@ extern "C" {
 double sage_microbench_units(int kind);
 int sage_microbench(int kind, int grid, int waves_per_simd, int iters, void* sink, size_t sink_bytes, void* stream);
 int sage_coexec(int mfma_kind, int valu_kind, int mode, int grid, int iters, void* sink, size_t sink_bytes, void* stream);
-int sage_period(int parts, int grid, int periods, void* sink, size_t sink_bytes, const void* src, size_t src_bytes, void* stream);
+int sage_period(int parts, int random_operands, int grid, int periods, void* sink, size_t sink_bytes, const void* src, size_t src_bytes, void* stream);
 #ifdef __cplusplus
 }
 #endif

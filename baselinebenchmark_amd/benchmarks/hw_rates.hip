@@ -197,11 +197,18 @@ __global__ void __launch_bounds__(512) coexec_kernel(int* sink, int iters, int m
 // prologue, epilogue, imbalance); with single pieces on, what each of them costs alone.
 // ---------------------------------------------------------------------------------------------
 template <int PARTS>
-__global__ void __launch_bounds__(512) period_kernel(int* sink, const uint8_t* src, int periods, float s, float c) {
+__global__ void __launch_bounds__(512) period_kernel(int* sink, const uint8_t* src, int periods, int random_operands, float s, float c) {
   constexpr bool MFMA = PARTS & 1, LDSF = PARTS & 2, VEC = PARTS & 4, DMA = PARTS & 8;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];   // 64 KB of fragments + 32 KB that the requests fill
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63, grp = wave >> 2;
-  for (int i = threadIdx.x; i < 65536 / 4; i += 512) reinterpret_cast<int*>(smem)[i] = i * 7 + 1;
+  // Operand bits: a regular low-entropy pattern, or hashed bytes (what quantised data looks like to the multipliers; the
+  // lowest bit of every byte cleared so that no FP8 byte is a NaN).  The instruction stream is the same either way.
+  auto hashed = [](unsigned x) {
+    x *= 2654435761u; x ^= x >> 15; x *= 2246822519u; x ^= x >> 13; x *= 3266489917u; x ^= x >> 16;
+    return (int)(x & 0xFEFEFEFEu);
+  };
+  for (int i = threadIdx.x; i < 65536 / 4; i += 512)
+    reinterpret_cast<int*>(smem)[i] = random_operands ? hashed(i + blockIdx.x * 16384) : i * 7 + 1;
   __syncthreads();
   const __amdgpu_buffer_rsrc_t rsrc =
       __builtin_amdgcn_make_buffer_rsrc((void*)(src + (size_t)(blockIdx.x & 7) * (1u << 20)), 0, 0x7fffffff, 0x00020000);
@@ -210,7 +217,11 @@ __global__ void __launch_bounds__(512) period_kernel(int* sink, const uint8_t* s
   v16f o[4];
   v4f osum = {0.f, 0.f, 0.f, 0.f};
   v8i ones;
-  for (int k = 0; k < 4; k++) q[k] = v4i{lane + k, 1, 2, 3};
+  for (int k = 0; k < 4; k++) {
+    q[k] = v4i{lane + k, 1, 2, 3};
+    if (random_operands)
+      for (int e = 0; e < 4; e++) q[k][e] = hashed(0x40000000u + ((blockIdx.x * 512 + threadIdx.x) * 4 + k) * 4 + e);
+  }
   for (int i = 0; i < 16; i++) bias[i] = 0x4B400000;
   for (int i = 0; i < 8; i++) ones[i] = (lane == 0 || lane == 32 || lane == 20 || lane == 52) ? 0x38383838 : 0;
   for (int k = 0; k < 4; k++) { acc[k] = bias; for (int i = 0; i < 16; i++) o[k][i] = 0.f; }
@@ -342,7 +353,7 @@ __global__ void __launch_bounds__(512) period_kernel(int* sink, const uint8_t* s
 }
 
 template <int PARTS>
-hipError_t launch_period(int* sink, const uint8_t* src, int grid, int periods, hipStream_t st) {
+hipError_t launch_period(int* sink, const uint8_t* src, int grid, int periods, int random_operands, hipStream_t st) {
   auto kern = period_kernel<PARTS>;
   static bool attr_done = false;
   if (!attr_done) {
@@ -350,7 +361,7 @@ hipError_t launch_period(int* sink, const uint8_t* src, int grid, int periods, h
     if (e != hipSuccess) return e;
     attr_done = true;
   }
-  kern<<<dim3(grid), dim3(512), 98304, st>>>(sink, src, periods, 0.999f, 0.001f);
+  kern<<<dim3(grid), dim3(512), 98304, st>>>(sink, src, periods, random_operands, random_operands ? 0.25f : 0.999f, 0.001f);
   return hipGetLastError();
 }
 
@@ -416,9 +427,13 @@ int sage_microbench(int kind, int grid, int waves_per_simd, int iters, void* sin
 // 3 = both.  Per iteration a wavefront issues 16 MFMAs, or 64 / 64 / 32 / 160 / 144 vector instructions.
 // The attention kernel's steady-state tile period as an instruction mix (see period_kernel): `parts` is a sum of 1 (MFMAs),
 // 2 (their A fragments come from LDS), 4 (the vector half), 8 (the global->LDS tile requests); supported: 1, 3, 4, 5, 7,
-// 11, 15.  `src` is device memory of at least grid MiB that the requests read.  The caller times the launch and divides
-// by `periods`.
-int sage_period(int parts, int grid, int periods, void* sink, size_t sink_bytes, const void* src, size_t src_bytes, void* stream) {
+// 11, 15.  random_operands 0: regular low-entropy operand bits; 1: hashed bytes in the fragments and the resident Q operand
+// (the scores then spread over a few binades below each tile's maximum, as attention scores do) -- the same
+// instructions on bits that toggle.
+// `src` is device memory of at least grid MiB that the requests read (fill it to match).  The caller times the launch
+// and divides by `periods`.
+int sage_period(int parts, int random_operands, int grid, int periods, void* sink, size_t sink_bytes, const void* src, size_t src_bytes,
+                void* stream) {
   using namespace sage;
   if (grid <= 0 || grid > 65535 || periods <= 0 || !sink || !src) return HWR_EINVAL;
   if (sink_bytes < (size_t)grid * 1024 * sizeof(int) || src_bytes < (size_t)grid << 20) return HWR_ESIZE;
@@ -427,13 +442,13 @@ int sage_period(int parts, int grid, int periods, void* sink, size_t sink_bytes,
   hipStream_t st = (hipStream_t)stream;
   hipError_t e;
   switch (parts) {
-    case 1: e = launch_period<1>(out, in, grid, periods, st); break;
-    case 3: e = launch_period<3>(out, in, grid, periods, st); break;
-    case 4: e = launch_period<4>(out, in, grid, periods, st); break;
-    case 5: e = launch_period<5>(out, in, grid, periods, st); break;
-    case 7: e = launch_period<7>(out, in, grid, periods, st); break;
-    case 11: e = launch_period<11>(out, in, grid, periods, st); break;
-    case 15: e = launch_period<15>(out, in, grid, periods, st); break;
+    case 1: e = launch_period<1>(out, in, grid, periods, random_operands != 0, st); break;
+    case 3: e = launch_period<3>(out, in, grid, periods, random_operands != 0, st); break;
+    case 4: e = launch_period<4>(out, in, grid, periods, random_operands != 0, st); break;
+    case 5: e = launch_period<5>(out, in, grid, periods, random_operands != 0, st); break;
+    case 7: e = launch_period<7>(out, in, grid, periods, random_operands != 0, st); break;
+    case 11: e = launch_period<11>(out, in, grid, periods, random_operands != 0, st); break;
+    case 15: e = launch_period<15>(out, in, grid, periods, random_operands != 0, st); break;
     default: return HWR_EINVAL;
   }
   return e == hipSuccess ? HWR_OK : HWR_ELAUNCH;

@@ -34,7 +34,7 @@ def lib() -> ctypes.CDLL:
         h.sage_coexec.restype = ctypes.c_int
         h.sage_coexec.argtypes = [ctypes.c_int] * 5 + [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
         h.sage_period.restype = ctypes.c_int
-        h.sage_period.argtypes = [ctypes.c_int] * 3 + [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
+        h.sage_period.argtypes = [ctypes.c_int] * 4 + [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
         _lib = h
     return _lib
 
@@ -143,27 +143,33 @@ PERIOD_PARTS = [
 
 def run_period(periods: int = 4000) -> list[dict]:
     """The attention kernel's steady-state tile period as an instruction mix (hw_rates.hip: period_kernel), one
-    workgroup per compute unit, wall clock per period, for the pieces alone and together."""
+    workgroup per compute unit, wall clock per period, for the pieces alone and together, on regular low-entropy operand
+    bits and on hashed ones (same instructions; the clock the part sustains depends on how many bits toggle)."""
     n_cu = torch.cuda.get_device_properties(0).multi_processor_count
     sink = torch.empty(n_cu * 1024, dtype=torch.int32, device="cuda")
-    src = torch.zeros(n_cu << 20, dtype=torch.uint8, device="cuda")
+    quiet = torch.zeros(n_cu << 20, dtype=torch.uint8, device="cuda")
+    noisy = torch.randint(0, 256, (n_cu << 20,), dtype=torch.uint8, device="cuda")
     stream = torch.cuda.current_stream().cuda_stream
     rows = []
     for parts, name in PERIOD_PARTS:
-        def launch():
-            check(lib().sage_period(parts, n_cu, periods, sink.data_ptr(), sink.numel() * 4, src.data_ptr(), src.numel(), stream))
-        launch()
-        torch.cuda.synchronize()
-        best = float("inf")
-        for _ in range(3):
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record(); launch(); e1.record()
+        ns = {}
+        for random_operands, src in ((0, quiet), (1, noisy)):
+            def launch():
+                check(lib().sage_period(parts, random_operands, n_cu, periods, sink.data_ptr(), sink.numel() * 4,
+                                        src.data_ptr(), src.numel(), stream))
+            launch()
             torch.cuda.synchronize()
-            best = min(best, e0.elapsed_time(e1) * 1e-3)
-        ns = best / periods * 1e9
+            best = float("inf")
+            for _ in range(3):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record(); launch(); e1.record()
+                torch.cuda.synchronize()
+                best = min(best, e0.elapsed_time(e1) * 1e-3)
+            ns[random_operands] = best / periods * 1e9
         # a period computes 256 query rows x 128 keys x head_dim 128 of both products
-        rows.append({"parts": parts, "name": name, "ns_per_period": ns,
-                     "chip_TOPS_if_the_whole_kernel_ran_like_this": 4.0 * 256 * 128 * 128 * n_cu / ns / 1e3})
+        rows.append({"parts": parts, "name": name, "ns_per_period": ns[0], "ns_per_period_random_operands": ns[1],
+                     "chip_TOPS_if_the_whole_kernel_ran_like_this": 4.0 * 256 * 128 * 128 * n_cu / ns[0] / 1e3,
+                     "chip_TOPS_random_operands": 4.0 * 256 * 128 * 128 * n_cu / ns[1] / 1e3})
     return rows
 
 
@@ -196,7 +202,9 @@ def main(argv=None) -> int:
           " 2176 matrix-pipe cycles per SIMD = 0.91 us at 2.4 GHz")
     for r in per:
         print(f"{r['name']:48s} {r['ns_per_period']:7.1f} ns per period   {r['chip_TOPS_if_the_whole_kernel_ran_like_this']:6.0f} TOPS "
-              f"({100 * r['chip_TOPS_if_the_whole_kernel_ran_like_this'] / 5033.2:.0f} % of peak) if a kernel were nothing but this")
+              f"({100 * r['chip_TOPS_if_the_whole_kernel_ran_like_this'] / 5033.2:.0f} % of peak) if a kernel were nothing but this;"
+              f" on random operand bits {r['ns_per_period_random_operands']:7.1f} ns, {r['chip_TOPS_random_operands']:6.0f} TOPS "
+              f"({100 * r['chip_TOPS_random_operands'] / 5033.2:.0f} %)")
     return 0
 
 

@@ -101,10 +101,15 @@ def test_hw_rate_microbenchmarks_run_and_are_plausible():
         assert r["both_s"] < 1.15 * (r["mfma_alone_s"] + r["valu_alone_s"]), r
     # the attention kernel's tile period as an instruction mix: the pieces alone and together.  The matrix pipe alone
     # needs 2176 cycles per period (0.9 us at 2.4 GHz); everything together lies between the longest piece and their sum
-    per = {r["parts"]: r["ns_per_period"] for r in hw_rates.run_period(periods=500)}
+    rows = hw_rates.run_period(periods=500)
+    per = {r["parts"]: r["ns_per_period"] for r in rows}
     assert set(per) == {p for p, _ in hw_rates.PERIOD_PARTS}
     assert 800 < per[1] < 1400 and per[3] >= 0.97 * per[1] and per[11] >= 0.97 * per[3], per
     assert max(per[3], per[4]) * 0.97 <= per[15] <= 1.1 * (per[11] + per[4]), per
+    # the same instructions on operand bits that toggle: never faster than on the regular pattern (beyond noise), and
+    # not slower than the clock range of the part allows
+    for r in rows:
+        assert 0.95 * r["ns_per_period"] <= r["ns_per_period_random_operands"] <= 2.0 * r["ns_per_period"], r
 
 
 @pytest.mark.gpu
