@@ -19,8 +19,14 @@
 //   * The INT32 accumulators start from the bit pattern of 1.5*2^23, so reading them as floats gives
 //     12582912 + dot exactly: the int->float conversion is folded into the one FMA that applies
 //     q_scale*k_scale and subtracts the running maximum.
-//   * The running maximum is only moved when it grows by more than kTau (lazy rescale); P is stored
-//     with a static 2^kPShift so that fp8's range [2^-9, 448] is used.
+//   * The running maximum is only moved when it grows by more than a threshold (lazy rescale).  The exact-exponential
+//     kernels store P with a static 2^pshift so that fp8's range [2^-9, 448] is used; the FP8 kernels without LSE or an
+//     explicit mask code P per (query row, 128-key tile) against the tile's own maximum (linear-mantissa e4m3 codes, no
+//     v_exp_f32) and hand the tile's power of two to the P.V MFMA as its E8M0 scale operand, so every tile uses the top
+//     of the code range however far it lies under the running maximum; their row sums come from the matrix pipe, unscaled
+//     per tile, and are folded into the running sum with one multiply by that power of two.
+//   * The tile decode (workgroup index -> head, tier, q-tile) divides by run-time values with host-made multiply-high
+//     dividers (sage_launch.h: FastDiv); the first K and V tiles are requested before the Q loads.
 //   * K/V tiles go global -> LDS directly (buffer_load ... lds, no registers): four slots per stream and
 //     requests two tile periods ahead for FP8 P.V, two slots and one period for FP16 P.V.  The raw q-tile of
 //     the variants that quantise their own Q and the V scales of the epilogue arrive the same way, and the
