@@ -32,4 +32,14 @@ extern "C" int sage_tile_timing(unsigned long long* out) {
   memset(sets, 0, sizeof(sets));
   return hipMemcpyToSymbol(HIP_SYMBOL(sage::g_tile_timing), sets, sizeof(sets)) == hipSuccess ? 0 : -1;
 }
+// Timing build only: copies the per-workgroup records of the last launch of a kernel of this translation unit (first
+// stamp, last stamp, XCC_ID << 32 | HW_ID, K tiles; four values each) for the first `count` workgroups to `out`.
+// Synchronises the device.  Returns the number of records copied or -1.
+extern "C" int sage_wg_timeline(unsigned long long* out, int count) {
+  if (count < 0) return -1;
+  if (count > sage::kTimelineMax) count = sage::kTimelineMax;
+  if (hipDeviceSynchronize() != hipSuccess) return -1;
+  if (hipMemcpyFromSymbol(out, HIP_SYMBOL(sage::g_wg_timeline), (size_t)count * 4 * sizeof(unsigned long long)) != hipSuccess) return -1;
+  return count;
+}
 #endif

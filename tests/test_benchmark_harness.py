@@ -124,7 +124,8 @@ def test_tile_timing_tool_reports_the_intervals_of_a_workgroup():
         pytest.skip("timing build absent (python -m baselinebenchmark_amd.build --tools)")
     code = ("from baselinebenchmark_amd.benchmarks import tile_timing as t\n"
             "rows, tiles = t.measure(2, 4, 4096, 128, True, launches=2)\n"
-            "import json; print(json.dumps({'rows': rows, 'tiles': tiles}))\n")
+            "line = t.timeline(2, 4, 4096, 128, True)\n"
+            "import json; print(json.dumps({'rows': rows, 'tiles': tiles, 'timeline': line}))\n")
     env = dict(os.environ, SAGE_MI355X_LIB=str(TIMING_LIB))
     res = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, env=env, cwd=ROOT, timeout=240)
     assert res.returncode == 0, res.stderr[-2000:]
@@ -145,6 +146,13 @@ def test_tile_timing_tool_reports_the_intervals_of_a_workgroup():
             continue
         assert len(vals) == 7 and all(v > 0 for v in vals), (name, vals)
         assert vals[4] > 0.5 * sum(vals), (name, vals)
+    # the launch seen from the compute units: every workgroup recorded once, on some compute unit, inside the launch span;
+    # 2 x 4 heads x 16 q-tiles with 2, 4, ..., 32 K tiles each
+    line = doc["timeline"]
+    assert line["workgroups"] == 128 and 1 <= line["compute_units"] <= 256
+    assert abs(line["k_tiles_per_cu"][0] * line["compute_units"] - 8 * 272) < 1e-6
+    assert line["inside_ns"][0] > 0 and line["gaps_ns"][1] >= 0 and line["after_last_ns"][1] == 0
+    assert line["inside_ns"][2] <= line["span_ns"] and len(line["xcd_finish_before_end_ns"]) <= 8
 
 
 @pytest.mark.gpu
