@@ -234,15 +234,21 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
           r0 += 1 << rs;
           if (r0 >= a.nqt) return;   // (a grid larger than the tile count: nothing to do)
         }
-        // Inside a round (32 consecutive workgroups of the XCD: one per compute unit) the LIGHTEST q-tile comes first.  The
-        // hardware hands out workgroups strictly in index order and round-robin over the XCD's four shader engines, so a
-        // free compute unit waits until every earlier workgroup has found a place in ITS engine: with the heaviest
-        // first, a round's workgroups finish in the reverse of the order in which their successors want their engines
-        // (measured: 6.4 us between two workgroups of a compute unit, against 1.5 us when all finish together); ascending
-        // cost inside a round makes compute units free up in dispatch order, round after round.  Ranges whose size is
-        // not a whole number of rounds (the last, lightest few) keep the plain order.
+        // Inside a round (32 consecutive workgroups of the XCD: one per compute unit) the order alternates: lightest
+        // q-tile first in even rounds, heaviest first in odd ones.  The hardware hands out workgroups strictly in index
+        // order and round-robin over the XCD's four shader engines, so a free compute unit waits until every earlier
+        // workgroup has found a place in ITS engine.  A round that starts on all compute units at once with ascending
+        // cost frees them in dispatch order; the next round, started one by one as they free up, has descending cost,
+        // so that it ends everywhere at the same time and the round after it starts together again -- which also
+        // keeps the compute units of the XCD in step on the K/V tiles they share through its L2.  (Measured on 2 x 32 heads
+        // of 16k rows, per hand-over of a compute unit from one workgroup to the next: 1.6 us this way; 6.4 us with the
+        // heaviest first in every round; 4.8 us with the lightest first in every round, whose compute units also drift
+        // apart and fetch 1.7 x the bytes into L2.)  Ranges
+        // whose size is not a whole number of rounds (the last, lightest few) keep the plain order.
         if (((hpx << rs) & 31) == 0) {
-          const int j = l & 31, hs = 5 - rs;   // position in the round; log2 of the heads a round covers
+          int j = l & 31;                      // position in the round
+          j = ((l >> 5) & 1) ? 31 - j : j;
+          const int hs = 5 - rs;               // log2 of the heads a round covers
           rank = r0 + ((1 << rs) - 1 - (j >> hs));
           s = x + 8 * (((l >> 5) << hs) + (j & ((1 << hs) - 1)));
         } else {
