@@ -88,12 +88,19 @@ def timeline(B, H, S, D, causal, dtype=torch.bfloat16, pv_mode="fp8", blkq=64, b
     fn = getattr(lib(), "sage_wg_timeline", None)
     if fn is None:
         raise SystemExit(f"{LIB_PATH} is not a timing build")
-    g = torch.Generator(device="cuda").manual_seed(0)
-    q, k, v = (torch.randn((B, H, S, D), dtype=dtype, device="cuda", generator=g) for _ in range(3))
-    _, _, ki, ks = sa.per_block_int8(q, k, BLKQ=blkq, BLKK=blkk)
-    for _ in range(6):
-        sa.forward_fused_q(q, ki, v, ks, is_causal=causal, pv_mode=pv_mode, BLKQ=blkq, BLKK=blkk)
-    n = B * H * ((S + 255) // 256)
+    if B == 0:      # the packed benchmark configuration (16 sequences of 512..32768 rows, 32 q-heads on 8 KV heads)
+        from baselinebenchmark_amd import workloads
+        wl = workloads.make("c4")
+        for _ in range(4):
+            sa.sageattn_varlen(wl.q, wl.k, wl.v, wl.cu_seqlens, wl.cu_seqlens, wl.max_seqlen, wl.max_seqlen, **wl.kwargs)
+        n = sum((L + 255) // 256 for L in wl.extra["lens"]) * wl.q.shape[1]
+    else:
+        g = torch.Generator(device="cuda").manual_seed(0)
+        q, k, v = (torch.randn((B, H, S, D), dtype=dtype, device="cuda", generator=g) for _ in range(3))
+        _, _, ki, ks = sa.per_block_int8(q, k, BLKQ=blkq, BLKK=blkk)
+        for _ in range(6):
+            sa.forward_fused_q(q, ki, v, ks, is_causal=causal, pv_mode=pv_mode, BLKQ=blkq, BLKK=blkk)
+        n = B * H * ((S + 255) // 256)
     buf = (ctypes.c_ulonglong * (4 * n))()
     got = fn(buf, n)
     if got <= 0:
@@ -131,14 +138,17 @@ def timeline(B, H, S, D, causal, dtype=torch.bfloat16, pv_mode="fp8", blkq=64, b
 def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--shapes", default="2x32x16384x128:1,2x32x16384x128:0,16x32x4096x128:1,64x32x1024x128:1",
-                    help="comma-separated BxHxSxD:causal")
+                    help="comma-separated BxHxSxD:causal (with --timeline also c4: the packed benchmark configuration)")
     ap.add_argument("--dump", default=None, help="with --timeline: folder that receives the raw per-workgroup records (.npy per shape)")
     ap.add_argument("--timeline", action="store_true",
                     help="per compute unit: time before the first workgroup, between workgroups, inside them, and idle at the end")
     args = ap.parse_args()
     for spec in args.shapes.split(","):
-        dims, causal = spec.split(":")
-        B, H, S, D = (int(x) for x in dims.split("x"))
+        if spec == "c4":     # (--timeline only) the packed benchmark configuration
+            dims, causal, B, H, S, D = "c4", "1", 0, 32, 0, 128
+        else:
+            dims, causal = spec.split(":")
+            B, H, S, D = (int(x) for x in dims.split("x"))
         if args.timeline:
             dump = None
             if args.dump:

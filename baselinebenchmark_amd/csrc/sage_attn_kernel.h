@@ -144,7 +144,7 @@ constexpr int kTimingSets = 256;
 static __device__ unsigned long long g_tile_timing[kTimingSets][48];
 // One record per workgroup of the last launch (the first kTimelineMax of them): first stamp, last stamp (ticks of the
 // chip-wide 100 MHz counter), where it ran (XCC_ID << 32 | HW_ID: compute unit, shader array and engine) and its K tiles.
-constexpr int kTimelineMax = 16384;
+constexpr int kTimelineMax = 65536;
 static __device__ unsigned long long g_wg_timeline[kTimelineMax][4];
 #define SAGE_PH(k) do { const long long t_ = __builtin_amdgcn_s_memrealtime(); if (ph_last) ph_sum[((k) + 3) & 3] += t_ - ph_last; ph_last = t_; if ((k) == 0) ph_n++; } while (0)
 #define SAGE_T(k, x) do { asm volatile("" : "+v"(x)); sage_ts[k] = __builtin_amdgcn_s_memrealtime(); } while (0)
