@@ -236,8 +236,6 @@ int attn_impl(const int8_t* q, const int8_t* k, const void* v_panels, const floa
   if ((qgroups > 1 || kgroups > 1) && cu_seqlens_q) return fail(SAGE_ENOTIMPL, "interleaved scales are not supported for packed batches");
   if (qgroups > 1 && qraw.ptr) return fail(SAGE_ENOTIMPL, "interleaved Q scales need the standalone Q quantiser (sage_quant_int8)");
   if (kgroups > 1 && blkk == 16) return fail(SAGE_ENOTIMPL, "interleaved K scales need blocks of 32, 64 or 128 keys");
-  if (kgroups > 1 && mask.ptr) return fail(SAGE_ENOTIMPL, "interleaved K scales cannot be combined with an explicit mask");
-  if (blkk == 16 && mask.ptr) return fail(SAGE_ENOTIMPL, "K scale blocks of 16 rows cannot be combined with an explicit mask");
   if (B == 0 || Hq == 0 || Sq == 0) return SAGE_OK;
   if (!out || (Skv > 0 && (!k || !v_panels || !k_scale))) return fail(SAGE_EINVAL, "null tensor pointer");
   if (!qraw.ptr && (!q || !q_scale)) return fail(SAGE_EINVAL, "null tensor pointer");
@@ -414,8 +412,8 @@ int sage_sageattn_masked(const void* q, const void* k, const void* v, void* out,
     return fail(SAGE_ENOTIMPL, "Q and K scale blocks must be 16, 32, 64 or 128 rows (got %d/%d)", blk_rows(blkq), blk_rows(blkk));
   if ((blk_groups(blkq) != 1 && blk_groups(blkq) != 8) || (blk_groups(blkk) != 1 && blk_groups(blkk) != 4))
     return fail(SAGE_ENOTIMPL, "Q scale blocks take SAGE_BLK_INTERLEAVE8, K scale blocks SAGE_BLK_INTERLEAVE4");
-  if (blk_groups(blkk) == 4 && (blk_rows(blkk) == 16 || attn_mask))
-    return fail(SAGE_ENOTIMPL, "interleaved K scales need blocks of 32, 64 or 128 keys and no explicit mask");
+  if (blk_groups(blkk) == 4 && blk_rows(blkk) == 16)
+    return fail(SAGE_ENOTIMPL, "interleaved K scales need blocks of 32, 64 or 128 keys");
   if (pv_mode != SAGE_PV_FP16 && pv_mode != SAGE_PV_FP8) return fail(SAGE_EINVAL, "pv_mode %d unknown", pv_mode);
   const int varlen = cu_seqlens_q != nullptr;
   if (varlen && (blk_groups(blkq) > 1 || blk_groups(blkk) > 1)) return fail(SAGE_ENOTIMPL, "interleaved scales are not supported for packed batches");

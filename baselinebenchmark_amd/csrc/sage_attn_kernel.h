@@ -619,7 +619,9 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
 #pragma unroll
         for (int r = 0; r < 16; r++) {
           const int n = n0 + 32 * nt + 8 * (r / 4) + 4 * h + (r % 4);
-          float sv = __builtin_fmaf(as_f(acc[nt][r]), sc[sci(nt, r)], -kBiasF * sc[sci(nt, r)]);
+          // (the bias comes off first, exactly: the product of the biased value would have to cancel against a
+          // rounded bias * scale, an error of half an ulp of that product -- 1e-3 at large scales)
+          float sv = (as_f(acc[nt][r]) - kBiasF) * sc[sci(nt, r)];
           const int64_t mi = mrow + (int64_t)min(n, Lk - 1) * a.m_sn;
           if constexpr (MASK == 1) sv = reinterpret_cast<const uint8_t*>(a.mask)[mi] ? sv : kNegInf;
           else sv = __builtin_fmaf(reinterpret_cast<const float*>(a.mask)[mi], a.mask_mult, sv);

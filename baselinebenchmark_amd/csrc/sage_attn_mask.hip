@@ -8,10 +8,15 @@
 namespace sage {
 
 hipError_t launch_attn_masked(const AttnArgs& a, int D, int pv, int grid, hipStream_t st) {
-#define SAGE_ATTN_M(DD, PVV, BNN) (a.mask_kind == 1 ? launch_one<DD, 8, BNN, PVV, false, false, 1>(a, grid, st) : launch_one<DD, 8, BNN, PVV, false, false, 2>(a, grid, st))
+  // K scale granularity: one scale per 32-key group or coarser, two per group (K blocks of 16 keys), or four interleaved
+  // scales per block -- the masked kernels turn the accumulators into scores element by element and look the scale of
+  // every element up, so the finer granularities only change that lookup.
+#define SAGE_ATTN_MK(DD, PVV, BNN, KS) (a.mask_kind == 1 ? launch_one<DD, 8, BNN, PVV, false, false, 1, KS>(a, grid, st) : launch_one<DD, 8, BNN, PVV, false, false, 2, KS>(a, grid, st))
+#define SAGE_ATTN_M(DD, PVV, BNN) (a.k_interleave ? SAGE_ATTN_MK(DD, PVV, BNN, 3) : a.blkk == 16 ? SAGE_ATTN_MK(DD, PVV, BNN, 2) : SAGE_ATTN_MK(DD, PVV, BNN, 1))
   if (D == 128) return pv ? SAGE_ATTN_M(128, 1, 128) : SAGE_ATTN_M(128, 0, 128);
   return pv ? SAGE_ATTN_M(64, 1, 128) : SAGE_ATTN_M(64, 0, 128);
 #undef SAGE_ATTN_M
+#undef SAGE_ATTN_MK
 }
 
 hipError_t launch_attn_k16(const AttnArgs& a, int D, int pv, bool causal, int grid, hipStream_t st) {

@@ -237,12 +237,10 @@ def forward(q, k, v, q_scale, k_scale, tensor_layout="HND", attn_mask=None, outp
     to [B, Hq, Sq, Skv] (sageattention_triton.py:92-105); not combinable with ``is_causal``.
     ``lse`` is base 2 (sageattention_triton.py:127-129) and an empty tensor unless requested.
     ``q_interleave=8`` / ``k_interleave=4``: q_scale / k_scale hold eight / four interleaved scales per block (see
-    per_block_int8); interleaved K scales cannot be combined with ``attn_mask``.
+    per_block_int8).
     """
     qflag = _check_interleave(q_interleave)
     kflag = _check_k_interleave(k_interleave, BLKK)
-    if kflag and attn_mask is not None:
-        raise NotImplementedError("interleaved K scales cannot be combined with attn_mask")
     for name, t in (("q", q), ("k", k)):
         if not isinstance(t, torch.Tensor) or not t.is_cuda or t.dtype != torch.int8 or not t.is_contiguous():
             raise TypeError(f"{name} must be contiguous GPU INT8")
@@ -288,7 +286,7 @@ def forward(q, k, v, q_scale, k_scale, tensor_layout="HND", attn_mask=None, outp
                                          _ptr(k_scale.contiguous()), _ptr(v_scale), _ptr(out),
                                          _ptr(lse if return_lse else None),
                                          B, Hq, Hkv, Sq, Skv, D, qsb, qsh, qsn, ksb, ksh, ksn, osb, osh, osn,
-                                         BLKQ | qflag, BLKK, pv, _dt(output_dtype), _ptr(m), kind, ms[0], ms[1], ms[2], ms[3],
+                                         BLKQ | qflag, BLKK | kflag, pv, _dt(output_dtype), _ptr(m), kind, ms[0], ms[1], ms[2], ms[3],
                                          _stream(q)))
         return out, lse
     check(lib().sage_attn_fwd(_ptr(q), _ptr(k), _ptr(panels), _ptr(q_scale.contiguous()), _ptr(k_scale.contiguous()),
@@ -383,7 +381,7 @@ def sageattn(q, k, v, tensor_layout="HND", is_causal=False, sm_scale=None, smoot
     ``max_seqlen_k`` bound the sequence lengths (derived from cu_seqlens, with one host synchronisation, when left
     out), and lse comes back as [Hq, total_q]; see sageattn_varlen, which this call is then identical to.
     ``q_interleave=8`` / ``k_interleave=4``: eight interleaved Q scales / four interleaved K scales per block (see
-    per_block_int8); fixed-length batches only, and interleaved K scales not together with ``attn_mask``.
+    per_block_int8); fixed-length batches only.
     """
     if qk_quant_dtype != "int8":
         raise NotImplementedError("only INT8 Q/K quantisation is implemented")
@@ -392,8 +390,6 @@ def sageattn(q, k, v, tensor_layout="HND", is_causal=False, sm_scale=None, smoot
     BLKQ, BLKK, pv_mode = _apply_recipe(quant_recipe, BLKQ, BLKK, pv_mode)
     qflag = _check_interleave(q_interleave)
     kflag = _check_k_interleave(k_interleave, BLKK)
-    if kflag and attn_mask is not None:
-        raise NotImplementedError("interleaved K scales cannot be combined with attn_mask")
     if cu_seqlens_q is not None or cu_seqlens_k is not None:
         if qflag or kflag:
             raise NotImplementedError("interleaved scales are not supported for packed batches")
@@ -440,7 +436,7 @@ def sageattn(q, k, v, tensor_layout="HND", is_causal=False, sm_scale=None, smoot
         m, kind, ms = _mask_args(attn_mask, B, Hq, Sq, Skv, q.device)
         check(lib().sage_sageattn_masked(_ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _ptr(ws), ws_bytes,
                                          B, Hq, Hkv, Sq, Skv, D, qsb, qsh, qsn, ksb, ksh, ksn, vsb, vsh, vsn, osb, osh, osn,
-                                         _dt(q.dtype), BLKQ | qflag, BLKK, float(D ** -0.5 if sm_scale is None else sm_scale),
+                                         _dt(q.dtype), BLKQ | qflag, BLKK | kflag, float(D ** -0.5 if sm_scale is None else sm_scale),
                                          0, int(bool(smooth_k)), pv, None, None, 0, 0,
                                          _ptr(m), kind, ms[0], ms[1], ms[2], ms[3], _stream(q)))
     else:

@@ -58,7 +58,7 @@ extern "C" {
  * every block of blkk = 32, 64 or 128 keys carries FOUR scales, scale t for the keys n of the block with (n % 8) / 2 == t
  * (keys 2t, 2t+1, 2t+8, 2t+9, ...): scale[(b*H + h)*ceil(S/blkk)*4 + block*4 + t].  In the transposed score tile a lane
  * holds keys of exactly two of the four groups per 32 keys, so the kernel applies two scales per lane and 32-key group.
- * Fixed-length batches only; not with an explicit mask. */
+ * Fixed-length batches only. */
 #define SAGE_BLK_INTERLEAVE4 0x200
 
 /* Rows of K/V covered by one V panel (see sage_prep_v). */
@@ -204,7 +204,8 @@ int sage_attn_fwd_qfused(const void* q, int q_dtype, double sm_scale,
  *   SAGE_MASK_BOOL     : logits of keys whose byte is 0 become -inf;
  *   SAGE_MASK_ADDITIVE : the fp32 value is added to the base-2 logits (q_scale already holds
  *                        sm_scale*log2(e), so the bias is in those units, as in the reference).
- * A row with no visible key yields out = 0 and LSE2 = -inf.  No causal flag and no packed mode here.
+ * A row with no visible key yields out = 0 and LSE2 = -inf.  Every K scale granularity is taken (blocks of 16 to 128 keys,
+ * SAGE_BLK_INTERLEAVE4).  No causal flag and no packed mode here.
  */
 int sage_attn_fwd_masked(const int8_t* q, const int8_t* k, const void* v_panels,
                          const float* q_scale, const float* k_scale, const float* v_scale,

@@ -141,7 +141,7 @@ def fp8_attention_model(q_int8, k_int8, v, q_scale, k_scale, tensor_layout="HND"
                 if is_causal:
                     dead |= keys[None, :] > rows_abs[:, None]
                 if masked:
-                    sv = _fma32(acc, sc, (-BIAS * sc).astype(np.float32))
+                    sv = ((acc - BIAS).astype(np.float32) * sc).astype(np.float32)   # bias off first (exact), one rounding
                     mk = mask[b, hq][:, n0:n1]
                     if mk.dtype == np.bool_:
                         dead |= ~mk

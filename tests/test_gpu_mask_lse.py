@@ -68,6 +68,52 @@ def test_forward_with_mask_matches_reference_formula(kind, pv, shape):
         assert (lse.cpu().double() - ref_lse).abs().max().item() < 3e-2
 
 
+@pytest.mark.parametrize("kind", ["bool_random", "additive_random", "additive_neg_inf"])
+@pytest.mark.parametrize("pv", ["fp16", "fp8"])
+@pytest.mark.parametrize("gran", [(128, 16, 1), (32, 64, 4), (64, 128, 4), (16, 32, 4)])
+@pytest.mark.parametrize("shape", [(1, 4, 2, 129, 70, 128), (2, 2, 1, 300, 391, 64)])
+def test_forward_with_mask_and_fine_k_scales(kind, pv, gran, shape):
+    """An explicit mask together with K scale blocks of 16 keys (the external (128, 16) recipe) and with four interleaved
+    K scales per block: against the formula with the scales expanded key by key.  (No counterpart in the reference,
+    whose forward has one K granularity: the masked kernels look the scale of every score up, so only the lookup
+    changes.)"""
+    B, Hq, Hkv, Sq, Skv, D = shape
+    blkq, blkk, ki4 = gran
+    g = torch.Generator().manual_seed(77 + D + Sq + blkk + ki4)
+    q = randn("HND", B, Hq, Sq, D, torch.float16, g)
+    k = randn("HND", B, Hkv, Skv, D, torch.float16, g, offset_std=1.0)
+    # keys of very different magnitude inside a block, so that a wrong scale lookup shows
+    k = k * (1.0 + 3.0 * (torch.arange(Skv) % 7 == 0).to(k.dtype))[None, None, :, None]
+    v = randn("HND", B, Hkv, Skv, D, torch.float16, g)
+    mask = _masks(kind, B, Hq, Sq, Skv, g)
+    qi, qs, ki, ks = sa.per_block_int8(q.to(DEV), k.to(DEV), BLKQ=blkq, BLKK=blkk, k_interleave=ki4)
+    out, lse = sa.forward(qi, ki, v.to(DEV), qs, ks, attn_mask=mask.to(DEV), return_lse=True, pv_mode=pv, BLKQ=blkq, BLKK=blkk,
+                          k_interleave=ki4)
+    torch.cuda.synchronize()
+    ref, ref_lse = oa.sage_reference(qi.cpu(), ki.cpu(), v, qs.cpu(), ks.cpu(), "HND", blkq, blkk, attn_mask=mask, k_interleave=ki4)
+    m = oa.metrics(out.cpu().float(), ref)
+    assert m["finite"]
+    if pv == "fp16":
+        assert m["rel_rmse"] < 2e-3
+        assert (lse.cpu().double() - ref_lse).abs().max().item() < 1e-3
+    else:
+        assert m["cosine"] >= 0.999 and m["rel_rmse"] < 5e-2
+        assert (lse.cpu().double() - ref_lse).abs().max().item() < 3e-2
+    # the one-call pipeline takes the same combination
+    full = sa.sageattn(q.to(DEV), k.to(DEV), v.to(DEV), attn_mask=mask.to(DEV), pv_mode=pv, BLKQ=blkq, BLKK=blkk, k_interleave=ki4)
+    torch.cuda.synchronize()
+    logits = torch.einsum("bhqd,bhkd->bhqk", q.double(), k.double().repeat_interleave(Hq // Hkv, 1)) * D ** -0.5
+    logits = logits.masked_fill(~mask, -float("inf")) if mask.dtype == torch.bool else logits + mask.double()
+    exact = torch.softmax(logits, -1) @ v.double().repeat_interleave(Hq // Hkv, 1)
+    assert oa.metrics(full.cpu().float(), exact)["cosine"] >= 0.999
+    # ... and without K smoothing it is the two steps above, bit for bit: the granularity reaches the pipeline's quantiser
+    # (boolean masks; an additive mask is in natural-log units there and in base-2 units for forward)
+    if mask.dtype == torch.bool:
+        plain = sa.sageattn(q.to(DEV), k.to(DEV), v.to(DEV), attn_mask=mask.to(DEV), pv_mode=pv, BLKQ=blkq, BLKK=blkk,
+                            k_interleave=ki4, smooth_k=False)
+        assert torch.equal(plain, out)
+
+
 def test_mask_broadcasts_without_being_materialised_and_accepts_half_bias():
     g = torch.Generator().manual_seed(11)
     B, Hq, Hkv, Sq, Skv, D = 2, 4, 2, 200, 333, 64
