@@ -138,9 +138,10 @@ void finish_attn_args(AttnArgs& a, bool causal) {
   a.div_range = a.div_last = make_fastdiv(1);
   // Per-XCD tile order (fixed-length batches whose heads and KV groups spread evenly over the eight XCDs): ranges of
   // R = 2^tier_shift consecutive q-tiles, R at most 32 and at most half of a head's q-tiles.  Causal problems with fewer than
-  // 16 q-tiles per compute unit keep the plain heaviest-first order: with so few rounds the balance of the last one
-  // matters more than locality (5 % on 4 x 32 heads of 4096 rows).
-  if (!packed && (heads & 7) == 0 && (groups & 7) == 0 && (!causal || (int64_t)a.nqt * (heads >> 3) >= 512)) {
+  // 16 q-tiles per compute unit keep the plain heaviest-first order -- with so few rounds the balance of the last one
+  // matters more than locality (1 x 32 heads of 4096 rows: 7 % slower with ranges) -- unless an XCD holds 16 heads or
+  // more and 8 q-tiles per compute unit (4 x 32 heads of 4096 rows: 2 % faster with ranges, 8 x 32 of 2048 rows 5 %).
+  if (!packed && (heads & 7) == 0 && (groups & 7) == 0 && (!causal || (int64_t)a.nqt * (heads >> 3) >= 512 || ((int64_t)a.nqt * (heads >> 3) >= 256 && (heads >> 3) >= 16))) {
     int shift = 5;
     while (shift > 0 && (2 << shift) > a.nqt) shift--;
     a.tier_shift = shift;
