@@ -335,6 +335,12 @@ namespace {
 // their sequence's statistics themselves (sage_quant.hip: prepass_small_kernel).
 constexpr int kSmallPrepassRows = 1024;
 constexpr int64_t kSmallPrepassElements = (int64_t)4 << 20;
+// ... and the element reads it makes: every K tile and every V panel re-reads its whole sequence, elements of K times
+// (K tiles + V panels per sequence).  Measured end to end against the six launches: 8 M reads (1 x 8 heads of 1024 rows,
+// head_dim 64, K blocks of 128) 30.0 against 31.2 us; 38 M (the same with K blocks of 16) 33.9 / 33.2; 100 M (1 x 32 heads
+// of 1024 rows, head_dim 128, K blocks of 64) 70 / 81; 302 M (the same with K blocks of 16) 68.7 / 54.2, and 8 x 8 heads of
+// 1024 rows at head_dim 64 with K blocks of 16, also 302 M, 88.9 / 50.1.
+constexpr int64_t kSmallPrepassReads = (int64_t)128 << 20;
 struct E2EWorkspace {
   size_t q_i8, k_i8, q_scale, k_scale, km, v_scale, panels, stat, plan, lse_off, total;
   int64_t qs_sh, ks_sh, panel_sh;
@@ -458,8 +464,10 @@ int sage_sageattn_masked(const void* q, const void* k, const void* v, void* out,
   if (no_keys) smooth_k = 0;
   // Short sequences: all K and V pre-passes in one launch (every workgroup computes the statistic its tile needs over
   // the whole sequence itself); otherwise six launches, the statistics in two stages.
-  const bool small_prepass = !varlen && !no_keys && Skv <= kSmallPrepassRows &&
-                             (int64_t)B * Hkv * Skv * D <= kSmallPrepassElements;
+  const int64_t k_elements = (int64_t)B * Hkv * Skv * D;
+  const int64_t rereads = (Skv + blk_rows(blkk) - 1) / blk_rows(blkk) + (Skv + kPanelRows - 1) / kPanelRows;
+  const bool small_prepass = !varlen && !no_keys && Skv <= kSmallPrepassRows && k_elements <= kSmallPrepassElements &&
+                             k_elements * rereads <= kSmallPrepassReads;
   if (small_prepass) {
     if (int rc2 = check_stride16("k", k_sb, k_sh, k_sn, 2, k)) return rc2;
     if (int rc2 = check_stride16("v", v_sb, v_sh, v_sn, 2, v)) return rc2;

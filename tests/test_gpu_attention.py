@@ -237,11 +237,15 @@ def test_lse_is_empty_unless_requested():
                                  ("HND", 1, 2, 1, 129, 1024, 128, torch.bfloat16, 32, 16),
                                  ("HND", 1, 2, 1, 40, 1025, 128, torch.bfloat16, 64, 128),     # one key too many: the six-launch path
                                  ("HND", 3, 2, 2, 77, 513, 64, torch.float16, 128, 32),
-                                 # the dearest case of the short path: 64 (batch, head) pairs x 64 K tiles of 16 keys at
-                                 # head_dim 64, exactly 4 M elements of K, every tile re-reading its whole sequence
+                                 # the dearest cases of the short path: 64 K tiles of 16 keys, every one re-reading its whole
+                                 # sequence of 1024 keys (2 x 8 heads at head_dim 64: 75 M element reads; limit 128 M), and
+                                 # exactly 4 M elements of K with K tiles of 64 keys (100 M reads)
+                                 ("HND", 2, 8, 8, 64, 1024, 64, torch.bfloat16, 64, 16),
+                                 ("HND", 1, 32, 32, 64, 1024, 128, torch.bfloat16, 64, 64),
+                                 # beyond the limit on re-reads (302 M): the six launches
                                  ("HND", 8, 8, 8, 64, 1024, 64, torch.bfloat16, 64, 16)])
 def test_one_call_on_short_sequences_equals_the_separate_calls_bitwise(cfg, pv, smooth):
-    """Up to 1024 keys (and 4 M elements of K) the one-call pipeline runs its K and V pre-passes as ONE launch, whose workgroups compute the K
+    """Up to 1024 keys (4 M elements of K, 128 M element reads) the one-call pipeline runs its K and V pre-passes as ONE launch, whose workgroups compute the K
     mean / V scale of their sequence themselves; the separate entry points use the two-stage statistics kernels.  Same
     int8 K, same scales, same panels: the attention output (and the LSE, which also sees the K mean) must be the same
     bits.  Sequence lengths off every block size, GQA, both layouts, the largest length of the short path and the first
