@@ -116,10 +116,13 @@ def time_attention_kernel(sa, S, w, iters: int):
     def launch():
         check(lib().sage_attn_fwd_qfused(S._ptr(q), S._dt(q.dtype), float(D ** -0.5), S._ptr(ki), S._ptr(panels), S._ptr(ks),
                                          S._ptr(vs), S._ptr(out), None, *args))
-    # (not part of the timed steps: as many untimed launches as the clocks need to settle after idle, about 25 ms)
-    for _ in range(20):
-        launch()
-    stream.synchronize()
+    # (not part of the timed steps: untimed launches until the clocks have settled after idle -- 50 ms of them, at least 20)
+    t_warm, n_warm = time.perf_counter(), 0
+    while n_warm < 20 or time.perf_counter() - t_warm < 0.05:
+        for _ in range(5):
+            launch()
+        stream.synchronize()
+        n_warm += 5
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record(stream)
     for _ in range(iters):
