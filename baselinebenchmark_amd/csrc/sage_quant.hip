@@ -19,7 +19,8 @@ namespace sage {
 // A lane owns 16 consecutive channels of a row (two 128-bit loads, one 128-bit store).
 // (km_lds: the K mean of this (batch, head) in LDS, D values in the input dtype, instead of a.km in global memory:
 // the fused pre-pass of short sequences computes it in the same workgroup.)
-template <int DT, int D>
+// UNIT: the multiplier is 1 (every K call; x * 1.0f is x, so leaving the product out changes no bit).
+template <int DT, int D, bool UNIT = false>
 __device__ __forceinline__ void quant_int8_tile(const QuantArgs& a, const int blkid, const int h, const int b, const u16* km_lds) {
   constexpr int TPR = D / 16;       // lanes per row
   constexpr int RPP = 256 / TPR;    // rows per pass
@@ -61,7 +62,7 @@ __device__ __forceinline__ void quant_int8_tile(const QuantArgs& a, const int bl
   // k - km is rounded to the input dtype (quant_per_block.py:53-54: the subtraction happens in torch, in
   // the tensor's dtype) once, while loading; both passes then see the rounded difference.
   auto smoothed = [&](u16 bits, int i) { return has_km ? from_f32<DT>(to_f32<DT>(bits) - kmv[i]) : bits; };
-  auto value = [&](u16 bits) { return to_f32<DT>(bits) * a.mult; };   // the fp32 value that is quantised
+  auto value = [&](u16 bits) { return UNIT ? to_f32<DT>(bits) : to_f32<DT>(bits) * a.mult; };   // the fp32 value that is quantised
 
   // Optional side output: the dot product of every (scaled) row with a per-(batch, kv-head) vector.
   // The one-call pipeline uses it with the K mean to return the LSE of the unsmoothed logits.
@@ -140,35 +141,37 @@ __device__ __forceinline__ void quant_int8_tile(const QuantArgs& a, const int bl
   const uint32_t sbits = __builtin_bit_cast(uint32_t, scale);
   const bool fast = ((sbits & 0x7fffffu) != 0x7fffffu) && scale < 1.0e30f;
 
+  // One wavefront-uniform branch around the whole second pass, not one per element (the scale is uniform over the tile,
+  // or, with interleaved scales, over a lane group: if any lane of the wavefront needs the true division, all take it --
+  // where the correction step applies, the two quotients are the same numbers).
+  auto quantise_rows = [&](auto quotient) __attribute__((always_inline)) {
 #pragma unroll
-  for (int p = 0; p < MAXP; p++) {
-    int r = p * RPP + tr;
-    if (r < rows) {
-      const u16* e = reinterpret_cast<const u16*>(raw[p]);
-      uint32_t packed[4] = {0, 0, 0, 0};
+    for (int p = 0; p < MAXP; p++) {
+      int r = p * RPP + tr;
+      if (r < rows) {
+        const u16* e = reinterpret_cast<const u16*>(raw[p]);
+        uint32_t packed[4] = {0, 0, 0, 0};
 #pragma unroll
-      for (int i = 0; i < 16; i++) {
-        const float x = value(e[i]);
-        float z;
-        if (fast) {
+        for (int i = 0; i < 16; i++) {
           // For |x| so small that the residual of the correction step is subnormal the quotient is
           // below 1e-13 in magnitude (scale >= 1e-12): whatever its last bits, it rounds to 0.
-          z = div_by_uniform(x, scale, rcp);
-        } else {
-          z = x / scale;
+          float z = quotient(value(e[i]));
+          z = z + __builtin_copysignf(0.5f, z);   // +0.5 for z >= 0 (incl. -0: -0.5 + -0 = -0.5 -> 0), else -0.5
+          int q = (int)z;  // truncation toward zero
+          packed[i >> 2] |= (uint32_t)(q & 0xff) << (8 * (i & 3));
         }
-        z = z + __builtin_copysignf(0.5f, z);   // +0.5 for z >= 0 (incl. -0: -0.5 + -0 = -0.5 -> 0), else -0.5
-        int q = (int)z;  // truncation toward zero
-        packed[i >> 2] |= (uint32_t)(q & 0xff) << (8 * (i & 3));
+        store_stream16(a.out + obase + (int64_t)(n0 + r) * a.o_sn + tc * 16, make_uint4(packed[0], packed[1], packed[2], packed[3]));
       }
-      store_stream16(a.out + obase + (int64_t)(n0 + r) * a.o_sn + tc * 16, make_uint4(packed[0], packed[1], packed[2], packed[3]));
     }
-  }
+  };
+  if (__builtin_amdgcn_ballot_w64(!fast) == 0) quantise_rows([&](float x) { return div_by_uniform(x, scale, rcp); });
+  else quantise_rows([&](float x) { return x / scale; });
 }
 
 template <int DT, int D>
 __global__ void __launch_bounds__(256) quant_int8_kernel(QuantArgs a) {
-  quant_int8_tile<DT, D>(a, blockIdx.x, blockIdx.y, blockIdx.z, nullptr);
+  if (a.mult == 1.0f) quant_int8_tile<DT, D, true>(a, blockIdx.x, blockIdx.y, blockIdx.z, nullptr);
+  else quant_int8_tile<DT, D, false>(a, blockIdx.x, blockIdx.y, blockIdx.z, nullptr);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -437,7 +440,7 @@ __global__ void __launch_bounds__(256) prepass_small_kernel(QuantArgs qa, PrepVA
       }
       __syncthreads();
     }
-    quant_int8_tile<DT, D>(qa, blockIdx.x, h, b, smooth ? km_l : nullptr);
+    quant_int8_tile<DT, D, true>(qa, blockIdx.x, h, b, smooth ? km_l : nullptr);   // (K: the multiplier is 1)
   } else {
     const int pidx = blockIdx.x - nk;
     if constexpr (PV == 1) {
