@@ -25,6 +25,12 @@
  * (0 a regular low-entropy pattern, 1 hashed bytes: the same instructions, but the multipliers, the register file and
  * LDS see bits that toggle, and the clock the part sustains differs).  What the schedule costs on the hardware before
  * masks, rescales, prologue, epilogue and imbalance.
+ *
+ * sage_period64: the same work per compute unit and period (256 query rows x 128 keys, head_dim 128) as an instruction mix
+ * for a design the attention kernel does NOT have: one wavefront per SIMD, 64 query rows per wavefront, so that every K / V
+ * fragment read from LDS feeds two MFMAs (half the fragment reads), matrix and vector work of neighbouring 64-key steps
+ * interleaved inside one instruction stream, output accumulators in the accumulation registers.  Whether that design
+ * would pay, measured before anyone writes the kernel.
  */
 #ifndef SAGE_HW_RATES_H
 #define SAGE_HW_RATES_H
@@ -39,6 +45,7 @@ extern "C" {
 double sage_microbench_units(int kind);
 int sage_microbench(int kind, int grid, int waves_per_simd, int iters, void* sink, size_t sink_bytes, void* stream);
 int sage_coexec(int mfma_kind, int valu_kind, int mode, int grid, int iters, void* sink, size_t sink_bytes, void* stream);
+int sage_period64(int random_operands, int grid, int periods, void* sink, size_t sink_bytes, const void* src, size_t src_bytes, void* stream);
 int sage_period(int parts, int random_operands, int grid, int periods, void* sink, size_t sink_bytes, const void* src, size_t src_bytes, void* stream);
 #ifdef __cplusplus
 }

@@ -352,6 +352,7 @@ __global__ void __launch_bounds__(512) period_kernel(int* sink, const uint8_t* s
   sink[blockIdx.x * 1024 + threadIdx.x] = result;
 }
 
+
 template <int PARTS>
 hipError_t launch_period(int* sink, const uint8_t* src, int grid, int periods, int random_operands, hipStream_t st) {
   auto kern = period_kernel<PARTS>;

@@ -33,6 +33,8 @@ def lib() -> ctypes.CDLL:
         h.sage_microbench.argtypes = [ctypes.c_int] * 4 + [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
         h.sage_coexec.restype = ctypes.c_int
         h.sage_coexec.argtypes = [ctypes.c_int] * 5 + [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
+        h.sage_period64.restype = ctypes.c_int
+        h.sage_period64.argtypes = [ctypes.c_int] * 3 + [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
         h.sage_period.restype = ctypes.c_int
         h.sage_period.argtypes = [ctypes.c_int] * 4 + [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
         _lib = h
@@ -141,6 +143,9 @@ PERIOD_PARTS = [
 ]
 
 
+ROWS64 = 64     # row key of the 64-rows-per-wavefront replica (sage_period64) in run_period's result
+
+
 def run_period(periods: int = 4000) -> list[dict]:
     """The attention kernel's steady-state tile period as an instruction mix (hw_rates.hip: period_kernel), one
     workgroup per compute unit, wall clock per period, for the pieces alone and together, on regular low-entropy operand
@@ -151,10 +156,14 @@ def run_period(periods: int = 4000) -> list[dict]:
     noisy = torch.randint(0, 256, (n_cu << 20,), dtype=torch.uint8, device="cuda")
     stream = torch.cuda.current_stream().cuda_stream
     rows = []
-    for parts, name in PERIOD_PARTS:
+    for parts, name in PERIOD_PARTS + [(ROWS64, "a design with 64 rows per wavefront (half the fragment reads)")]:
         ns = {}
         for random_operands, src in ((0, quiet), (1, noisy)):
             def launch():
+                if parts == ROWS64:
+                    check(lib().sage_period64(random_operands, n_cu, periods, sink.data_ptr(), sink.numel() * 4,
+                                              src.data_ptr(), src.numel(), stream))
+                    return
                 check(lib().sage_period(parts, random_operands, n_cu, periods, sink.data_ptr(), sink.numel() * 4,
                                         src.data_ptr(), src.numel(), stream))
             launch()

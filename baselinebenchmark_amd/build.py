@@ -82,13 +82,17 @@ def build_tools(verbose: bool = True) -> list[Path]:
     """Builds what the benchmark tools need and the drop-in library does not contain: the instrumented twin of the
     library (tile_timing), the hardware-rate micro-benchmarks (hw_rates) and the C++ benchmark driver."""
     out = [build(verbose, timing=True)]
-    obj = BENCH / "hw_rates.o"
-    # (the attention kernels' scheduling flags: the micro-benchmarks reproduce their instruction streams)
-    res = subprocess.run([_hipcc(), *FLAGS, *EXTRA_FLAGS["sage_attn.hip"], "-c", str(BENCH / "hw_rates.hip"), "-o", str(obj)],
-                         capture_output=True, text=True)
-    if res.returncode != 0:
-        raise RuntimeError(f"hipcc failed for hw_rates.hip:\n{res.stderr}")
-    out.append(_link([obj], HWRATES_LIB, verbose))
+    objs = []
+    # (the attention kernels' scheduling flags: the micro-benchmarks reproduce their instruction streams; the replica of
+    # the 64-rows-per-wavefront design keeps its scores in vector registers, see hw_rates_rows64.hip)
+    for name, extra in (("hw_rates", []), ("hw_rates_rows64", ["-mllvm", "-amdgpu-mfma-vgpr-form"])):
+        obj = BENCH / f"{name}.o"
+        res = subprocess.run([_hipcc(), *FLAGS, *EXTRA_FLAGS["sage_attn.hip"], *extra, "-c", str(BENCH / f"{name}.hip"), "-o", str(obj)],
+                             capture_output=True, text=True)
+        if res.returncode != 0:
+            raise RuntimeError(f"hipcc failed for {name}.hip:\n{res.stderr}")
+        objs.append(obj)
+    out.append(_link(objs, HWRATES_LIB, verbose))
     src = BENCH / "sage_bench.cpp"
     if src.exists():
         cmd = [_hipcc(), "-O2", "-std=c++17", "-x", "hip", "--offload-arch=gfx950", str(src), "-I", str(CSRC.parent.parent / "include"),
